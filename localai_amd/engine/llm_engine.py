@@ -35,6 +35,7 @@ import torch
 from .. import ops
 from ..gguf import GGUFReader  # noqa: F401 (re-exported for callers)
 from ..models.hf_checkpoint import open_model
+from ..models import model_class
 from ..models.decoder import DecoderModel, ForwardBatch, TPInfo
 from ..native import core
 from ..tokenizer import Tokenizer
@@ -113,6 +114,14 @@ class EngineConfig:
     # waves -> 121; gpurun_out/r5_fc_base.log vs r5_fc_ra.log)
     grammar_run_ahead: bool = dataclasses.field(
         default_factory=lambda: os.environ.get("LOCALAI_AMD_GRAMMAR_RUN_AHEAD", "1") == "1")
+    # serving precision: "bfloat16" (bf16 GEMMs and activations; fp32 residual, norms, scores) or
+    # "float32" (everything in true 32-bit) for the model families that implement it
+    dtype: str = "bfloat16"
+    # models with per-sequence state beside the paged K/V: slots of the state pool (0: max_num_seqs)
+    state_slots: int = 0
+    # size the KV pool to exactly max_kv_tokens (no spare blocks): replaying a recorded schedule
+    # against the pool it was recorded for
+    kv_pool_exact: bool = False
 
 
 @dataclass
@@ -191,9 +200,24 @@ class LLMEngine:
         if cfg.lora_adapters:
             from ..models.lora import LoraSet
             lora = LoraSet(cfg.lora_adapters)
-        self.model = DecoderModel(self.reader, self.device, tp=tp, max_pos=cfg.context_size, rope_overrides=ro,
-                                  lora=lora)
+        cls = model_class(self.reader.architecture)
+        if cls is DecoderModel:
+            if cfg.dtype not in ("bfloat16", "bf16"):
+                raise ValueError(f"{self.reader.architecture}: this model family serves in bfloat16 only")
+            self.model = DecoderModel(self.reader, self.device, tp=tp, max_pos=cfg.context_size, rope_overrides=ro,
+                                      lora=lora)
+        else:
+            dt = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+                  "fp32": torch.float32}.get(cfg.dtype)
+            if dt is None:
+                raise ValueError(f"unknown serving dtype {cfg.dtype!r}")
+            self.model = cls(self.reader, self.device, tp=tp, max_pos=cfg.context_size, rope_overrides=ro, lora=lora,
+                             dtype=dt)
         self.hp = self.model.hp
+        # per-sequence state (convolution tails, recurrent state) lives in a slot pool the native
+        # scheduler hands out; a cached K/V prefix carries no such state, so prefix reuse is off
+        self.stateful = bool(getattr(self.model, "stateful", False))
+        self.state_slots = (cfg.state_slots or cfg.max_num_seqs) if self.stateful else 0
         self.vocab = core.Vocab(self.tokenizer.pieces)
         self.gvocab = core.GrammarVocab(self.tokenizer.pieces, sorted(self.tokenizer.eog))
         self._eog_list = sorted(self.tokenizer.eog)
@@ -225,7 +249,7 @@ class LLMEngine:
                 raise ValueError(f"mmproj projects to {self.clip.out_dim}, the LLM embeds {self.hp.n_embd}")
         self.ctx = cfg.context_size
         bs = cfg.block_size
-        if self.device.type == "cuda":
+        if self.device.type == "cuda" and isinstance(self.model, DecoderModel):
             # legacy path (LOCALAI_AMD_TILE_GEMM=0): prefill / big decode batches run hipBLASLt on
             # bf16 copies, materialised before any graph capture.  The default path multiplies the
             # quantised weights directly (gemm_q.hip) and keeps no copy -- except for formats the
@@ -244,13 +268,14 @@ class LLMEngine:
             num_blocks = int(nb.item())
         if faults.hit("kv_alloc"):
             raise faults.InjectedFault("hipMalloc failed for the KV cache (injected fault): out of memory")
-        self.kv = self.model.new_kv_cache(num_blocks, bs)
+        self.kv = self.model.new_kv_cache(num_blocks, bs, self.state_slots)
         self.drafter = None
         if cfg.draft_model:
             self.drafter = DraftModel(cfg.draft_model, self.device, cfg.draft_max_seqs, self.ctx, self.hp.n_vocab,
                                       max_batched_tokens=cfg.max_batched_tokens)
         self.sched = core.Scheduler(num_blocks, bs, cfg.max_num_seqs, cfg.max_batched_tokens, self.ctx,
-                                    cfg.prefix_cache, 1 if (cfg.use_graphs and self.device.type == "cuda") else 0)
+                                    cfg.prefix_cache and not self.stateful,
+                                    1 if (cfg.use_graphs and self.device.type == "cuda") else 0, self.state_slots)
         self.max_blocks = (self.ctx + bs - 1) // bs
         self.requests: Dict[int, Request] = {}
         self._inbox: "queue.Queue" = queue.Queue()
@@ -345,7 +370,7 @@ class LLMEngine:
         log.info("materialised %.2f GB of bf16 weight copies", need / 2**30)
 
     def _kv_block_bytes(self) -> int:
-        return 2 * self.hp.n_layer * self.model.Hkv * self.cfg.block_size * self.model.Dh * 2
+        return self.model.kv_bytes_per_token() * self.cfg.block_size
 
     def _kv_blocks_wanted(self) -> int:
         cfg = self.cfg
@@ -357,6 +382,8 @@ class LLMEngine:
         cfg = self.cfg
         bpb = self._kv_block_bytes()
         want = self._kv_blocks_wanted()
+        if cfg.kv_pool_exact and cfg.max_kv_tokens:
+            return (cfg.max_kv_tokens + cfg.block_size - 1) // cfg.block_size
         if self.device.type == "cuda":
             free, total = torch.cuda.mem_get_info(self.device)
             free += torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
@@ -762,7 +789,7 @@ class LLMEngine:
         if len(r.prompt) >= self.ctx:
             r.callback(Event(finished=True, finish_reason="error", error="prompt exceeds context"))
             return
-        if r.params.prompt_cache_path and self.tp.world == 1:
+        if r.params.prompt_cache_path and self.tp.world == 1 and not self.stateful:
             n = self._pcache.ensure_loaded(self, r.params.prompt_cache_path)
             if n:
                 log.info("prompt cache %s: %d tokens of KV restored", r.params.prompt_cache_path, n)
@@ -847,6 +874,87 @@ class LLMEngine:
                     self.fatal_error = str(e)
                     raise
 
+    # ------------------------------------------------------------------ schedule replay
+    def replay_step(self, entries: Sequence[tuple], end: Sequence[int] = ()) -> Optional[torch.Tensor]:
+        """One step of a recorded schedule, run by the engine's scheduler, KV pool and kernels but
+        with the batch given instead of planned: entries = [(sequence id, next tokens, wanted)],
+        where `wanted` lists the places among these tokens whose logits are asked for.  A sequence
+        is admitted at its first entry (KV blocks and, for stateful models, a state slot), may rest
+        for any number of steps, and is released when listed in `end`.  Nothing is sampled.  All
+        entries run as ONE batch: a model with `mixed_batches` takes prompt portions and single
+        decoded tokens in one forward; the others run the portions through the prefill kernels and
+        the single tokens through the decode kernels of the same step.  Returns fp32 logits
+        [wanted rows, vocab] in the order of entries and wanted places (None if nothing is wanted).
+        Not to be mixed with add_request()/step() traffic on the same engine."""
+        if self.requests:
+            raise RuntimeError("replay_step: the engine is serving requests")
+        for rid, toks, _ in entries:
+            toks = [int(t) for t in toks]
+            if not toks:
+                raise ValueError("replay_step: an entry without tokens")
+            if self.sched.has(rid):
+                self.sched.extend(rid, toks)
+            else:
+                self.sched.add(rid, toks, 0)
+        logits = None
+        if entries:
+            plan = self.sched.schedule_explicit([(rid, len(toks)) for rid, toks, _ in entries])
+            ids = [int(i) for i in plan["p_ids"]]
+            cu = plan["p_cu"]
+            first = {rid: int(cu[k]) for k, rid in enumerate(ids)}
+            rows = [first[rid] + int(w) for rid, toks, want in entries for w in want]
+            for rid, toks, want in entries:
+                if any(not 0 <= int(w) < len(toks) for w in want):
+                    raise ValueError("replay_step: a wanted place outside the entry's tokens")
+            logits = self._replay_forward(plan, rows)
+            self.metrics["prompt_tokens"] += int(cu[-1])
+            self.metrics["steps"] += 1
+        for rid in end:
+            self.sched.finish(rid)
+        return logits
+
+    def _replay_forward(self, plan, rows: List[int]) -> Optional[torch.Tensor]:
+        cu, qlens, dec = plan["p_cu"], plan["p_qlen"], plan["p_decode"]
+        n = len(qlens)
+        nc = int(n - dec.sum())          # chunks first, single-token continuations after them
+        gpu = self.device.type == "cuda"
+        idx = (lambda r: self._dev(np.array(r, dtype=np.int64)) if r else None)
+        if getattr(self.model, "mixed_batches", False):
+            fb = ForwardBatch(tokens=self._dev(plan["p_tokens"]), pos=self._dev(plan["p_pos"]),
+                              slots=self._dev(plan["p_slots"]), decode=False, block_tables=self._dev(plan["p_bt"]),
+                              cu_q=self._dev(cu), ctx_lens=self._dev(plan["p_ctx"]), logits_idx=idx(rows),
+                              sslots=self._dev(plan["p_sslot"]),
+                              row_seq=self._dev(np.repeat(np.arange(n, dtype=np.int32), qlens)))
+            if not rows:
+                self.model.forward(fb, self.kv)
+                return None
+            return self.model.forward(fb, self.kv).float()
+        # two kernels families, one step: portions through prefill, single tokens through decode
+        tp = int(cu[nc])
+        out = {}
+        if nc:
+            prow = [r for r in rows if r < tp]
+            fb = ForwardBatch(tokens=self._dev(plan["p_tokens"][:tp]), pos=self._dev(plan["p_pos"][:tp]),
+                              slots=self._dev(plan["p_slots"][:tp]), decode=False,
+                              block_tables=self._dev(plan["p_bt"][:nc]), cu_q=self._dev(cu[:nc + 1]),
+                              ctx_lens=self._dev(plan["p_ctx"][:nc]),
+                              tiles=ops.prefill_tiles(qlens[:nc].tolist(), self.device) if gpu else None,
+                              logits_idx=idx(prow))
+            if prow:
+                lg = self.model.forward(fb, self.kv).float()
+                out.update({r: lg[k] for k, r in enumerate(prow)})
+            else:
+                self.model.forward(fb, self.kv)
+        if n > nc:
+            lens = plan["p_ctx"][nc:]
+            fb = ForwardBatch(tokens=self._dev(plan["p_tokens"][tp:]), pos=self._dev(plan["p_pos"][tp:]),
+                              slots=self._dev(plan["p_slots"][tp:]), decode=True,
+                              block_tables=self._dev(plan["p_bt"][nc:]), seq_lens=self._dev(lens),
+                              max_len=int(lens.max()))
+            lg = self.model.forward(fb, self.kv).float()
+            out.update({r: lg[r - tp] for r in rows if r >= tp})
+        return torch.stack([out[r] for r in rows]) if rows else None
+
     def _dev(self, a: np.ndarray) -> torch.Tensor:
         t = torch.from_numpy(np.ascontiguousarray(a))
         if self.device.type == "cuda":
@@ -881,9 +989,13 @@ class LLMEngine:
         fb = ForwardBatch(
             tokens=self._dev(tokens), pos=self._dev(plan["p_pos"]), slots=self._dev(plan["p_slots"]),
             decode=False, block_tables=self._dev(plan["p_bt"]), cu_q=self._dev(cu), ctx_lens=self._dev(plan["p_ctx"]),
-            tiles=ops.prefill_tiles(qlens.tolist(), self.device) if self.device.type == "cuda" else None,
+            tiles=(ops.prefill_tiles(qlens.tolist(), self.device)
+                   if self.device.type == "cuda" and isinstance(self.model, DecoderModel) else None),
             logits_idx=self._dev(np.array(rows, dtype=np.int64)) if rows else None,
             inject_idx=inj_idx, inject_rows=inj_rows)
+        if self.stateful:
+            fb.sslots = self._dev(plan["p_sslot"])
+            fb.row_seq = self._dev(np.repeat(np.arange(len(ids), dtype=np.int32), qlens))
         self.metrics["prompt_tokens"] += int(cu[-1])
         if not rows:
             self.model.forward(fb, self.kv)  # intermediate chunk: KV only
@@ -1013,6 +1125,8 @@ class LLMEngine:
         prompt is still prefilling."""
         if not self.requests or len(self.requests) > self.SPEC_MAX_BATCH or self.sched.num_waiting:
             return 0
+        if self.stateful:   # rejected draft tokens would have advanced the per-sequence state
+            return 0
         k = 0
         for r in self.requests.values():
             p = r.params
@@ -1092,9 +1206,11 @@ class LLMEngine:
         B = len(ids)
         tok, pos, slots, lens, bt = plan["d_tokens"], plan["d_pos"], plan["d_slots"], plan["d_lens"], plan["d_bt"]
         Bp = len(tok)
+        self._cur_sslot = plan["d_sslot"]
         if not (self.cfg.use_graphs and self.device.type == "cuda"):
             fb = ForwardBatch(tokens=self._dev(tok), pos=self._dev(pos), slots=self._dev(slots), decode=True,
-                              block_tables=self._dev(bt), seq_lens=self._dev(lens), max_len=int(plan["d_maxlen"]))
+                              block_tables=self._dev(bt), seq_lens=self._dev(lens), max_len=int(plan["d_maxlen"]),
+                              sslots=self._dev(plan["d_sslot"]) if self.stateful else None)
             logits = self.model.forward(fb, self.kv)
             self._sample_and_emit(ids, logits[:B])
             return
@@ -1393,6 +1509,7 @@ class LLMEngine:
         h["pos"][:] = torch.from_numpy(pos)
         h["slots"][:] = torch.from_numpy(slots)
         h["lens"][:] = torch.from_numpy(lens)
+        h["sslot"][:] = torch.from_numpy(self._cur_sslot)
         nb = bt.shape[1]
         h["bt"][:, :nb] = torch.from_numpy(bt)
         h["step"][0] = 0
@@ -1521,7 +1638,7 @@ class LLMEngine:
         layout = [("tokens", Bp), ("pos", Bp), ("slots", Bp), ("lens", Bp), ("bt", Bp * MB), ("step", 1),
                   ("prm", prm_words), ("bias_rows", cap), ("bias_cols", cap), ("bias_vals", cap), ("bias_n", 1),
                   ("mu", Bp), ("phist", Bp * PL), ("pcnt", Bp), ("phl", Bp), ("pcap", Bp), ("pen", Bp * 3),
-                  ("pnl", Bp), ("gslot", Bp)]
+                  ("pnl", Bp), ("gslot", Bp), ("sslot", Bp)]
         total = sum(n for _, n in layout)
         host_block = torch.zeros(total, dtype=torch.int32).pin_memory()
         dev_block = torch.zeros(total, dtype=torch.int32, device=dev)
@@ -1543,6 +1660,7 @@ class LLMEngine:
         st["slots"].fill_(-1)
         st["lens"].fill_(1)
         st["gslot"].fill_(-1)
+        st["sslot"].fill_(-1)
         st["host"], st["host_block"], st["dev_block"] = host, host_block, dev_block
 
         st["prm_np"] = np.zeros(Bp, dtype=ops.SAMPLE_ROW_DTYPE)
@@ -1550,9 +1668,8 @@ class LLMEngine:
         st["next"] = torch.zeros(Bp, dtype=torch.int32, device=dev)
         st["hist"] = torch.zeros(K, Bp, dtype=torch.int32, device=dev)
         fb = ForwardBatch(tokens=st["tokens"], pos=st["pos"], slots=st["slots"], decode=True, block_tables=st["bt"],
-                          seq_lens=st["lens"], max_len=self.ctx)
-        ws = ops.decode_workspace(Bp, self.model.Hq, self.model.Hkv, self.model.Dh, self.ctx, dev,
-                                  self.cfg.block_size)
+                          seq_lens=st["lens"], max_len=self.ctx, sslots=st["sslot"] if self.stateful else None)
+        ws = self.model.decode_workspace(Bp, self.ctx, self.cfg.block_size)
         bs = self.cfg.block_size
         if tp_local:
             vl = self.model.vocab_local
@@ -2112,7 +2229,7 @@ class LLMEngine:
         tail = r.stream.flush() if (flush and r.stream is not None) else b""
         p = r.params
         if p.prompt_cache_path and not p.prompt_cache_ro and r.n_gen > 0 and self.tp.world == 1 \
-                and self.sched.has(r.id):
+                and self.sched.has(r.id) and not self.stateful:
             try:
                 toks = self.sched.tokens(r.id)
                 keep = len(toks) - 1 if p.prompt_cache_all else r.n_prompt  # tokens whose KV exists

@@ -220,6 +220,10 @@ class ForwardBatch:
     logits_idx: Optional[torch.Tensor] = None  # rows to project to logits (None: all)
     inject_idx: Optional[torch.Tensor] = None  # prefill rows whose embedding is given (images)
     inject_rows: Optional[torch.Tensor] = None  # [n, n_embd] f32
+    # models with per-sequence state (short-convolution tails): the state slot of every sequence
+    # (decode: of every row; -1 = none) and, for prompt batches, the sequence index of every row
+    sslots: Optional[torch.Tensor] = None      # [nseq] i32 (decode: [B])
+    row_seq: Optional[torch.Tensor] = None     # prefill: [T] i32
 
 
 class KVCache:
@@ -238,9 +242,32 @@ class KVCache:
         self.v = [torch.zeros(num_blocks, n_kv, block_size // 8, head_dim, 8, dtype=dtype, device=device)
                   for _ in range(n_layer)]
 
+    state = None        # per-layer state pools [slots, rows, channels] (KVCache.layered), else None
+    state_slots = 0
+
     @staticmethod
     def bytes_per_block(n_layer, n_kv, block_size, head_dim, dtype_bytes=2):
         return 2 * n_layer * n_kv * block_size * head_dim * dtype_bytes
+
+    @classmethod
+    def layered(cls, specs, num_blocks: int, block_size: int, device, dtype=torch.bfloat16,
+                state_slots: int = 0) -> "KVCache":
+        """Pools for layers that differ in shape: specs[i] = (kv heads, key width, value width,
+        state shape or None).  K and V pages are both row-major [num_blocks, heads, block_size,
+        width] (ops.kv_pages: the layout ops.shortconv_kv writes and ops.attn_mix reads); layers
+        with a state shape get a pool [state_slots, *shape] beside them, indexed by the scheduler's
+        state slots.  Slots are never cleared: a kernel reads of a slot only what lies at
+        positions >= 0 of the sequence that holds it."""
+        kv = cls.__new__(cls)
+        kv.num_blocks, kv.block_size = num_blocks, block_size
+        kv.k = [ops.kv_pages(num_blocks, g, block_size, dk, dtype, device) for g, dk, _, _ in specs]
+        kv.v = [ops.kv_pages(num_blocks, g, block_size, dv, dtype, device) for g, _, dv, _ in specs]
+        kv.state_slots = state_slots
+        kv.state = None
+        if state_slots > 0:
+            kv.state = [torch.zeros(state_slots, *st, dtype=dtype, device=device) if st is not None else None
+                        for _, _, _, st in specs]
+        return kv
 
 
 @dataclass
@@ -547,8 +574,17 @@ class DecoderModel:
         return ops.QWeight.from_raw(raw, gt, shape, self.device)
 
     # --------------------------------------------------------------------------- forward
-    def new_kv_cache(self, num_blocks: int, block_size: int) -> KVCache:
+    stateful = False        # no per-sequence state beside the paged K/V
+    mixed_batches = False   # prompt chunks and decode rows run as two forwards
+
+    def new_kv_cache(self, num_blocks: int, block_size: int, state_slots: int = 0) -> KVCache:
         return KVCache(self.hp.n_layer, num_blocks, self.Hkv, block_size, self.Dh, self.device)
+
+    def kv_bytes_per_token(self) -> int:
+        return 2 * self.hp.n_layer * self.Hkv * self.Dh * 2
+
+    def decode_workspace(self, Bp: int, ctx: int, block_size: int):
+        return ops.decode_workspace(Bp, self.Hq, self.Hkv, self.Dh, ctx, self.device, block_size)
 
     def _row_parallel_out(self, p: ops.Partial, bias) -> ops.Partial:
         if self.tp.world == 1:

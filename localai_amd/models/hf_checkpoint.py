@@ -63,9 +63,27 @@ QUANT_MODES = {"bnb_4bit": "q4_k_m", "xpu_4bit": "q4_k_m", "q4_k_m": "q4_k_m", "
                "bnb_8bit": "q8_0", "xpu_8bit": "q8_0", "q8_0": "q8_0"}
 
 
+# checkpoint directories whose config.json names ONE design under "architecture" and lists its
+# layers one by one ("layers": [{type, mixer, mlp}, ...]): design name -> engine architecture
+LAYERED_ARCH_OF = {"Suganex": "suganex"}
+
+
+def layered_architecture(path: str) -> str:
+    """Engine architecture of a layer-list checkpoint directory ("" when it is not one)."""
+    try:
+        with open(os.path.join(path, "config.json")) as f:
+            c = json.load(f)
+    except (OSError, ValueError):
+        return ""
+    a = c.get("architecture")
+    return LAYERED_ARCH_OF.get(a, "") if isinstance(a, str) and isinstance(c.get("layers"), list) else ""
+
+
 def open_model(path: str, quantization: str = ""):
     """GGUF file, HF checkpoint directory or pre-GGUF ggjt v3 file -> reader with the GGUFReader
     interface.  `quantization`: load-time quantisation of an HF checkpoint (QUANT_MODES)."""
+    if is_hf_checkpoint(path) and layered_architecture(path):
+        return LayeredCheckpointReader(path)
     if is_hf_checkpoint(path):
         return HFCheckpointReader(path, quantization=quantization)
     from .ggml_legacy import GGJTReader, is_ggjt
@@ -100,6 +118,57 @@ def _llama3_rope_freqs(rs: dict, head_dim: int, theta: float) -> np.ndarray:
             smooth = (old / wl - lo) / (hi - lo)
             out.append(1.0 / ((1 - smooth) / factor + smooth))
     return np.asarray(out, dtype=np.float32)
+
+
+class LayeredCheckpointReader:
+    """config.json + model.safetensors of a layer-list design, behind the GGUFReader interface:
+    `architecture`, `kv` (general.* and a numeric tokenizer: such checkpoints ship no vocabulary,
+    token i is the piece "<i>") and `tensors` under the checkpoint's own names (raw little-endian
+    payloads, bf16 / f32 / i32 as stored).  `config` is the parsed config.json: the model class
+    (models.MODEL_CLASSES) reads every size and constant from it."""
+
+    def __init__(self, path: str):
+        self.path = path
+        with open(os.path.join(path, "config.json")) as f:
+            self.config: Dict[str, Any] = json.load(f)
+        self.arch = layered_architecture(path)
+        if not self.arch:
+            raise ValueError(f"{path}: unknown layer-list design {self.config.get('architecture')!r}")
+        self.kv: Dict[str, Any] = {"general.architecture": self.arch,
+                                   "general.name": os.path.basename(os.path.normpath(path))}
+        self.tensors: Dict[str, GGUFTensor] = {}
+        from safetensors import safe_open
+        import torch
+        for fn in sorted(glob.glob(os.path.join(path, "*.safetensors"))):
+            with safe_open(fn, framework="pt") as f:
+                for k in f.keys():
+                    t = f.get_tensor(k)
+                    if t.dtype in (torch.int32, torch.int64):
+                        arr, gt = t.to(torch.int32).contiguous().numpy(), GGMLType.I32
+                    else:
+                        arr, gt = HFCheckpointReader._np(t)
+                    arr = np.ascontiguousarray(arr)
+                    data = arr.view(np.uint8).reshape(-1)
+                    self.tensors[k] = GGUFTensor(k, tuple(int(x) for x in arr.shape), int(gt), 0, data.nbytes, data)
+        n_vocab = int(self.config.get("vocab") or 0)
+        self.kv["tokenizer.ggml.model"] = "numeric"
+        self.kv["tokenizer.ggml.tokens"] = [f"<{i}>" for i in range(n_vocab)]
+
+    @property
+    def architecture(self) -> str:
+        return self.arch
+
+    def get(self, key: str, default=None):
+        return self.kv.get(key, default)
+
+    def close(self):
+        self.tensors = {}
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
 
 
 class HFCheckpointReader:

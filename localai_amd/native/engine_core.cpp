@@ -234,14 +234,20 @@ struct SeqInfo {
   int n_gen = 0;
   bool running = false;
   int64_t order = 0;
+  int sslot = -1;  // state slot (models with per-sequence recurrent / convolution state), -1: none
 };
 
 class Scheduler {
  public:
+  // state_slots > 0: the model keeps a fixed-size state per sequence beside its paged KV (short
+  // convolution tails, recurrent state).  A sequence holds one slot of that pool from admission
+  // until it finishes or is preempted; admission waits while no slot is free.
   Scheduler(int num_blocks, int block_size, int max_num_seqs, int max_batched_tokens, int max_model_len,
-            bool prefix_cache, int decode_bucket_pad)
+            bool prefix_cache, int decode_bucket_pad, int state_slots = 0)
       : bm_(num_blocks, block_size, prefix_cache), max_seqs_(max_num_seqs), max_tok_(max_batched_tokens),
-        max_len_(max_model_len), pad_(decode_bucket_pad) {}
+        max_len_(max_model_len), pad_(decode_bucket_pad), n_sslots_(state_slots) {
+    for (int i = state_slots - 1; i >= 0; --i) sslot_free_.push_back(i);
+  }
 
   BlockManager& blocks() { return bm_; }
 
@@ -263,10 +269,23 @@ class Scheduler {
     auto it = seqs_.find(id);
     if (it == seqs_.end()) return;
     bm_.free_seq(id);
+    release_sslot(it->second);
     running_.erase(std::remove(running_.begin(), running_.end(), id), running_.end());
     waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), id), waiting_.end());
     seqs_.erase(it);
   }
+
+  // More input tokens for a live sequence (a prompt that arrives in portions): they count as
+  // prompt, not as generated tokens.
+  void extend(int64_t id, const std::vector<int32_t>& toks) {
+    SeqInfo& s = seqs_.at(id);
+    for (int32_t t : toks) s.toks.push_back(t);
+    s.n_prompt += (int)toks.size();
+  }
+
+  int num_free_state_slots() const { return (int)sslot_free_.size(); }
+  int state_slot(int64_t id) const { return seqs_.at(id).sslot; }
+  int n_computed(int64_t id) const { return seqs_.at(id).n_computed; }
 
   void append(int64_t id, int32_t tok) {
     SeqInfo& s = seqs_.at(id);
@@ -339,7 +358,6 @@ class Scheduler {
 
     // ---- 2. prefill chunks under the token budget
     int budget = max_tok_;
-    struct Chunk { int64_t id; int start; int n; };
     std::vector<Chunk> chunks;
     for (int64_t id : pre_cont) {
       if (budget <= 0) break;
@@ -352,9 +370,11 @@ class Scheduler {
     while (!waiting_.empty() && budget > 0 && (int)running_.size() < max_seqs_) {
       const int64_t id = waiting_.front();
       SeqInfo& s = seqs_.at(id);
+      if (n_sslots_ > 0 && sslot_free_.empty()) break;  // every state slot is held by a running sequence
       const int cached = bm_.allocate(id, s.toks, (int)s.toks.size());
       if (cached < 0) break;  // out of KV blocks: wait for running sequences to finish
       waiting_.pop_front();
+      take_sslot(s);
       s.n_computed = cached;
       s.running = true;
       running_.push_back(id);
@@ -373,57 +393,7 @@ class Scheduler {
     // ---- 3. pack device inputs
     py::dict out;
     const int bs = bm_.block_size();
-    {
-      const int np = (int)chunks.size();
-      int T = 0, maxb = 1;
-      for (auto& c : chunks) {
-        T += c.n;
-        maxb = std::max(maxb, bm_.blocks_for(c.start + c.n));
-      }
-      py::array_t<int64_t> ids(np);
-      py::array_t<int32_t> tok(T), pos(T), slot(T), cu(np + 1), ctx(np), qlen(np), bt({np, maxb});
-      py::array_t<uint8_t> last(np);
-      auto* pid = ids.mutable_data();
-      auto* pt = tok.mutable_data();
-      auto* pp = pos.mutable_data();
-      auto* ps = slot.mutable_data();
-      auto* pc = cu.mutable_data();
-      auto* pctx = ctx.mutable_data();
-      auto* pq = qlen.mutable_data();
-      auto* pb = bt.mutable_data();
-      auto* pl = last.mutable_data();
-      int o = 0;
-      pc[0] = 0;
-      for (int i = 0; i < np; ++i) {
-        const Chunk& c = chunks[i];
-        SeqInfo& s = seqs_.at(c.id);
-        pid[i] = c.id;
-        const std::vector<int> tab = bm_.table(c.id);
-        for (int j = 0; j < c.n; ++j) {
-          const int p = c.start + j;
-          pt[o] = s.toks[p];
-          pp[o] = p;
-          ps[o] = tab[p / bs] * bs + (p % bs);
-          ++o;
-        }
-        pc[i + 1] = o;
-        pctx[i] = c.start + c.n;
-        pq[i] = c.n;
-        pl[i] = (c.start + c.n == (int)s.toks.size()) ? 1 : 0;
-        for (int b = 0; b < maxb; ++b) pb[i * maxb + b] = b < (int)tab.size() ? tab[b] : 0;
-        s.n_computed = c.start + c.n;
-        bm_.commit(c.id, s.toks, s.n_computed);
-      }
-      out["p_ids"] = ids;
-      out["p_tokens"] = tok;
-      out["p_pos"] = pos;
-      out["p_slots"] = slot;
-      out["p_cu"] = cu;
-      out["p_ctx"] = ctx;
-      out["p_qlen"] = qlen;
-      out["p_bt"] = bt;
-      out["p_last"] = last;
-    }
+    pack_chunks(chunks, out);
     {
       const int B = (int)dec.size();
       int Bp = B;
@@ -435,12 +405,13 @@ class Scheduler {
         maxlen = std::max(maxlen, n);
       }
       py::array_t<int64_t> ids(B);
-      py::array_t<int32_t> tok(Bp), pos(Bp), slot(Bp), lens(Bp), bt({Bp, maxb});
+      py::array_t<int32_t> tok(Bp), pos(Bp), slot(Bp), lens(Bp), sslot(Bp), bt({Bp, maxb});
       auto* pid = ids.mutable_data();
       auto* pt = tok.mutable_data();
       auto* pp = pos.mutable_data();
       auto* ps = slot.mutable_data();
       auto* pl = lens.mutable_data();
+      auto* pss = sslot.mutable_data();
       auto* pb = bt.mutable_data();
       for (int i = 0; i < Bp; ++i) {
         if (i < B) {
@@ -453,6 +424,7 @@ class Scheduler {
           pp[i] = p;
           ps[i] = tab[p / bs] * bs + (p % bs);
           pl[i] = p + 1;
+          pss[i] = s.sslot;
           for (int b = 0; b < maxb; ++b) pb[i * maxb + b] = b < (int)tab.size() ? tab[b] : 0;
           s.n_computed = p + 1;
           bm_.commit(id, s.toks, s.n_computed);
@@ -461,6 +433,7 @@ class Scheduler {
           pp[i] = 0;
           ps[i] = -1;
           pl[i] = 1;
+          pss[i] = -1;
           for (int b = 0; b < maxb; ++b) pb[i * maxb + b] = 0;
         }
       }
@@ -469,10 +442,47 @@ class Scheduler {
       out["d_pos"] = pos;
       out["d_slots"] = slot;
       out["d_lens"] = lens;
+      out["d_sslot"] = sslot;
       out["d_bt"] = bt;
       out["d_maxlen"] = maxlen;
     }
     out["preempted"] = preempted;
+    return out;
+  }
+
+  // Replay of a recorded schedule: run exactly `n` more tokens of each listed sequence this step
+  // (a sequence not listed rests), in ONE batch.  Sequences are admitted at their first entry;
+  // nothing is preempted: a plan that does not fit the KV pool or the state slots is an error.
+  // Chunks come first and single-token continuations (decode rows, p_decode = 1) last, each
+  // group in the order given.  Packs the same arrays as schedule()'s prefill part.
+  py::dict schedule_explicit(const std::vector<std::pair<int64_t, int>>& entries) {
+    std::vector<Chunk> chunks, singles;
+    for (auto& e : entries) {
+      const int64_t id = e.first;
+      SeqInfo& s = seqs_.at(id);
+      if (!s.running) {
+        if (n_sslots_ > 0 && sslot_free_.empty()) throw std::runtime_error("schedule_explicit: no free state slot");
+        const int cached = bm_.allocate(id, s.toks, (int)s.toks.size());
+        if (cached < 0) throw std::runtime_error("schedule_explicit: out of KV blocks");
+        waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), id), waiting_.end());
+        take_sslot(s);
+        s.n_computed = cached;
+        s.running = true;
+        running_.push_back(id);
+      }
+      const int n = e.second;
+      if (n < 1 || s.n_computed + n > (int)s.toks.size())
+        throw std::invalid_argument("schedule_explicit: a sequence has fewer tokens left than the step asks for");
+      if (!bm_.ensure(id, s.n_computed + n)) throw std::runtime_error("schedule_explicit: out of KV blocks");
+      (n == 1 && s.n_computed > 0 ? singles : chunks).push_back({id, s.n_computed, n});
+    }
+    const int n_chunks = (int)chunks.size();
+    chunks.insert(chunks.end(), singles.begin(), singles.end());
+    py::dict out;
+    pack_chunks(chunks, out);
+    py::array_t<uint8_t> dec((int)chunks.size());
+    for (int i = 0; i < (int)chunks.size(); ++i) dec.mutable_data()[i] = i >= n_chunks ? 1 : 0;
+    out["p_decode"] = dec;
     return out;
   }
 
@@ -484,6 +494,77 @@ class Scheduler {
   }
 
  private:
+  struct Chunk { int64_t id; int start; int n; };
+
+  // Device inputs of a batch of prompt chunks: tokens, positions, KV slots, per-sequence query
+  // ranges / context lengths / block tables / state slots.  Marks the chunks computed.
+  void pack_chunks(const std::vector<Chunk>& chunks, py::dict& out) {
+    const int bs = bm_.block_size();
+    const int np = (int)chunks.size();
+    int T = 0, maxb = 1;
+    for (auto& c : chunks) {
+      T += c.n;
+      maxb = std::max(maxb, bm_.blocks_for(c.start + c.n));
+    }
+    py::array_t<int64_t> ids(np);
+    py::array_t<int32_t> tok(T), pos(T), slot(T), cu(np + 1), ctx(np), qlen(np), sslot(np), bt({np, maxb});
+    py::array_t<uint8_t> last(np);
+    auto* pid = ids.mutable_data();
+    auto* pt = tok.mutable_data();
+    auto* pp = pos.mutable_data();
+    auto* ps = slot.mutable_data();
+    auto* pc = cu.mutable_data();
+    auto* pctx = ctx.mutable_data();
+    auto* pq = qlen.mutable_data();
+    auto* pss = sslot.mutable_data();
+    auto* pb = bt.mutable_data();
+    auto* pl = last.mutable_data();
+    int o = 0;
+    pc[0] = 0;
+    for (int i = 0; i < np; ++i) {
+      const Chunk& c = chunks[i];
+      SeqInfo& s = seqs_.at(c.id);
+      pid[i] = c.id;
+      const std::vector<int> tab = bm_.table(c.id);
+      for (int j = 0; j < c.n; ++j) {
+        const int p = c.start + j;
+        pt[o] = s.toks[p];
+        pp[o] = p;
+        ps[o] = tab[p / bs] * bs + (p % bs);
+        ++o;
+      }
+      pc[i + 1] = o;
+      pctx[i] = c.start + c.n;
+      pq[i] = c.n;
+      pss[i] = s.sslot;
+      pl[i] = (c.start + c.n == (int)s.toks.size()) ? 1 : 0;
+      for (int b = 0; b < maxb; ++b) pb[i * maxb + b] = b < (int)tab.size() ? tab[b] : 0;
+      s.n_computed = c.start + c.n;
+      bm_.commit(c.id, s.toks, s.n_computed);
+    }
+    out["p_ids"] = ids;
+    out["p_tokens"] = tok;
+    out["p_pos"] = pos;
+    out["p_slots"] = slot;
+    out["p_cu"] = cu;
+    out["p_ctx"] = ctx;
+    out["p_qlen"] = qlen;
+    out["p_sslot"] = sslot;
+    out["p_bt"] = bt;
+    out["p_last"] = last;
+  }
+
+  void take_sslot(SeqInfo& s) {
+    if (n_sslots_ <= 0 || s.sslot >= 0) return;
+    s.sslot = sslot_free_.back();
+    sslot_free_.pop_back();
+  }
+  void release_sslot(SeqInfo& s) {
+    if (s.sslot < 0) return;
+    sslot_free_.push_back(s.sslot);
+    s.sslot = -1;
+  }
+
   static int next_bucket(int b) {
     if (b < 8) return b * 2;
     if (b < 64) return b + 8;
@@ -498,6 +579,7 @@ class Scheduler {
   void preempt(int64_t id) {
     SeqInfo& s = seqs_.at(id);
     bm_.free_seq(id);
+    release_sslot(s);
     s.n_computed = 0;
     s.running = false;
     running_.erase(std::remove(running_.begin(), running_.end(), id), running_.end());
@@ -505,7 +587,8 @@ class Scheduler {
   }
 
   BlockManager bm_;
-  int max_seqs_, max_tok_, max_len_, pad_;
+  int max_seqs_, max_tok_, max_len_, pad_, n_sslots_;
+  std::vector<int> sslot_free_;
   std::unordered_map<int64_t, SeqInfo> seqs_;
   std::deque<int64_t> waiting_;
   std::vector<int64_t> running_;
@@ -542,8 +625,15 @@ PYBIND11_MODULE(_la_core, m) {
       .def_property_readonly("hit_tokens", &BlockManager::hits)
       .def_property_readonly("query_tokens", &BlockManager::queries);
   py::class_<Scheduler>(m, "Scheduler")
-      .def(py::init<int, int, int, int, int, bool, int>())
+      .def(py::init<int, int, int, int, int, bool, int, int>(), py::arg("num_blocks"), py::arg("block_size"),
+           py::arg("max_num_seqs"), py::arg("max_batched_tokens"), py::arg("max_model_len"), py::arg("prefix_cache"),
+           py::arg("decode_bucket_pad"), py::arg("state_slots") = 0)
       .def("add", &Scheduler::add)
+      .def("extend", &Scheduler::extend)
+      .def("schedule_explicit", &Scheduler::schedule_explicit)
+      .def("state_slot", &Scheduler::state_slot)
+      .def("n_computed", &Scheduler::n_computed)
+      .def_property_readonly("num_free_state_slots", &Scheduler::num_free_state_slots)
       .def("finish", &Scheduler::finish)
       .def("append", &Scheduler::append)
       .def("schedule", &Scheduler::schedule, py::arg("lookahead") = 1, py::arg("defer_decode") = false)

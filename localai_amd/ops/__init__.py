@@ -28,6 +28,19 @@ _LIB = None
 _LIB_LOCK = threading.Lock()
 
 FMT_Q8_0, FMT_Q4_K, FMT_Q6_K, FMT_BF16 = 8, 12, 14, 30
+FMT_F32 = 0   # dense fp32 [N, K] (models served in true 32-bit: library SGEMM, no reduced-precision mode)
+
+
+_REQUIRED: Optional[Tuple[str, ...]] = None
+
+
+def require_kernels(files: Optional[Sequence[str]]) -> None:
+    """Before the first lib(): the kernel sources this process will launch (a model class's
+    `kernel_sources`).  Where the whole library is built it is loaded as always; on a checkout
+    without it only these sources are compiled (ops/_build.build_subset) instead of every GEMM
+    family.  None: no restriction."""
+    global _REQUIRED
+    _REQUIRED = tuple(sorted(set(files))) if files else None
 
 
 def lib():
@@ -41,8 +54,12 @@ def lib():
         from . import _build
         path = _build.LIB
         alt = os.environ.get("LOCALAI_AMD_KLIB")  # an A/B build of the same sources (_build.build_variant)
+        partial = False
         if alt:
             path = _build.HERE / alt
+        elif not path.exists() and _REQUIRED and not os.environ.get("LOCALAI_AMD_REBUILD"):
+            path = _build.build_subset(_REQUIRED)
+            partial = True
         elif not path.exists() or os.environ.get("LOCALAI_AMD_REBUILD"):
             _build.build()
         L = ctypes.CDLL(str(path))
@@ -102,6 +119,10 @@ def lib():
             "la_bsgemm_glu": [I, P, P, P, I, P, P, P, I, I, I, P, I, I, P, I, I, I, P],
             "la_bsmoe": [I, I, P, I, I, I, P, P, I, P, I, I, I, P, P, I, LNG, I, I, P],
             "la_decode_advance": [P, P, P, P, P, P, I, I, I, P, I, P, P, P],
+            "la_shortconv_kv": [I, I, P, I, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, P, P, P, I, I, P],
+            "la_attn_mix_rows": [I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
+            "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
+            "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
             "la_img_resample_v_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P, P, P, P, P],
         }
@@ -116,12 +137,13 @@ def lib():
                 continue
             fn.argtypes = args
             fn.restype = I
-        if missing:
+        if missing and not partial:
             import warnings
             warnings.warn(f"{path.name} lacks {', '.join(missing)}: rebuild it (python -c 'from localai_amd.ops "
                           f"import _build; _build.build()')")
-        L.la_gemm_scales_bytes.argtypes = [I, I]
-        L.la_gemm_scales_bytes.restype = LNG
+        if hasattr(L, "la_gemm_scales_bytes"):
+            L.la_gemm_scales_bytes.argtypes = [I, I]
+            L.la_gemm_scales_bytes.restype = LNG
         gv = os.environ.get("LOCALAI_AMD_GEMV_VARIANT")
         if gv is not None:
             _check(L.la_gemv_variant(int(gv)), "la_gemv_variant")
@@ -226,6 +248,18 @@ class QWeight:
             return QWeight(FMT_BF16, N, K, (None, None, None, None), ref=w.float())
         wb = w.to(torch.bfloat16).contiguous()
         return QWeight(FMT_BF16, N, K, (wb.view(torch.uint8).view(N, K * 2), None, None, None))
+
+    @staticmethod
+    def from_f32(w: torch.Tensor) -> "QWeight":
+        """Dense fp32 weight for the 32-bit serving mode (linear_multi: x fp32 @ W^T by the library SGEMM)."""
+        N, K = w.shape
+        if w.device.type != "cuda":
+            return QWeight(FMT_F32, N, K, (None, None, None, None), ref=w.float())
+        wf = w.float().contiguous()
+        return QWeight(FMT_F32, N, K, (wf.view(torch.uint8).view(N, K * 4), None, None, None))
+
+    def f32(self) -> torch.Tensor:
+        return self.planes[0].view(torch.float32).view(self.N, self.K)
 
     def ptrs(self):
         return [_ptr(p) for p in self.planes]
@@ -998,8 +1032,14 @@ def linear_multi(x: torch.Tensor, ws: Sequence[QWeight], bias: Optional[torch.Te
     if not x.is_cuda:
         y = torch.cat([x.float() @ w.dequant_f32().t() for w in ws], -1)
         return Partial(y.to(torch.bfloat16) if force == "bf16" else y.unsqueeze(0), bias)
+    if x.dtype == torch.float32 and all(w.fmt == FMT_F32 for w in ws):
+        # 32-bit serving mode: the library SGEMM (torch keeps TF32-style modes off unless asked)
+        y = torch.matmul(x, ws[0].f32().t()) if len(ws) == 1 else torch.cat([torch.matmul(x, w.f32().t()) for w in ws], -1)
+        return Partial(y.unsqueeze(0), bias)
     if x.dtype != torch.bfloat16 or not x.is_contiguous():
         raise ValueError("linear: x must be contiguous bf16")
+    if any(w.fmt == FMT_F32 for w in ws):
+        raise ValueError("linear: fp32 weights take fp32 activations")
     skinny_ok = all(w.K % 256 == 0 for w in ws)
     use_skinny = (M <= SKINNY_MAX_M and skinny_ok) if force is None else force == "skinny"
     tile_ok = TILE_GEMM and all(w.tile_ok for w in ws)
@@ -1311,6 +1351,7 @@ def rope_kv(qkv: Partial, pos: torch.Tensor, slots: Optional[torch.Tensor], cos_
 
 
 ACT_SWIGLU, ACT_GELU, ACT_GELU_QUICK, ACT_GEGLU = 0, 1, 2, 3
+ACT_RELU2 = 4   # max(x, 0)^2
 GLU_ACTS = (ACT_SWIGLU, ACT_GEGLU)  # gate|up sources of width 2F
 
 
@@ -1324,6 +1365,8 @@ def act(src: Partial, F: int, mode: int, out: Optional[torch.Tensor] = None) -> 
             y = torch.nn.functional.gelu(x[:, :F], approximate="tanh") * x[:, F:2 * F]
         elif mode == ACT_GELU:
             y = torch.nn.functional.gelu(x, approximate="tanh")
+        elif mode == ACT_RELU2:
+            y = torch.relu(x).square()
         else:
             y = x * torch.sigmoid(1.702 * x)
         return y.to(torch.bfloat16)
@@ -1668,6 +1711,219 @@ def _attn_ref_prefill(q, kc, vc, cu_q, ctx_lens, bt, scale, softcap=0.0, window=
         p = torch.softmax(sc, -1)
         out[a:b] = torch.einsum("hql,hld->hqd", p, v).transpose(0, 1).to(q.dtype)
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# Short causal convolution on q | k | v + paged K/V append; score-modifier attention
+# ---------------------------------------------------------------------------------------
+
+def kv_pages(nblk: int, G: int, BS: int, D: int, dtype=torch.bfloat16, device=None) -> torch.Tensor:
+    """Row-major K or V pages [blocks, G, BS, D] (the layout shortconv_kv writes and attn_mix reads)."""
+    return torch.zeros(nblk, G, BS, D, dtype=dtype, device=device)
+
+
+def shortconv_kv(u: torch.Tensor, w: torch.Tensor, Cq: int, Ck: int, Cv: int, row_seq: torch.Tensor,
+                 cu_q: torch.Tensor, pos: torch.Tensor, slots: torch.Tensor, sslot: torch.Tensor,
+                 state: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 vfirst_in: Optional[torch.Tensor] = None, vfirst_out: Optional[torch.Tensor] = None,
+                 lam: Optional[torch.Tensor] = None, single: bool = False) -> torch.Tensor:
+    """Depthwise causal convolution over time (w [C, taps] fp32, C = Cq + Ck + Cv) on the first C
+    columns of the projection rows u [T, >= C]; rows of one sequence portion are consecutive
+    (row_seq [T] -> sequence, cu_q [nseq + 1] row ranges, pos [T] positions).  What precedes a
+    portion comes from state[sslot[seq]] ([slots, taps - 1, C]: the last taps - 1 projected rows),
+    zeros before position 0; the state then advances to the end of the portion.  Returns q [T, Cq];
+    k and v go to the paged pools ([blocks, G, BS, Dk / Dv]) at `slots` (-1: nowhere), v first mixed
+    as (1 - lam) v + lam vfirst_in when given; vfirst_out receives the unmixed v (fp32 [T, Cv]).
+    single: every sequence brings one row (decode batches): one fused launch."""
+    T = u.shape[0]
+    C = Cq + Ck + Cv
+    taps = w.shape[1]
+    nseq = cu_q.shape[0] - 1
+    G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    Dv = v_cache.shape[3]
+    if (w.shape[0] != C or u.shape[1] < C or Ck != G * Dk or Cv != G * Dv or state.shape[1:] != (max(taps - 1, 0), C)
+            or row_seq.shape[0] != T or pos.shape[0] != T or slots.shape[0] != T or sslot.shape[0] != nseq):
+        raise ValueError("shortconv_kv: operand shapes do not fit")
+    if single and nseq != T:
+        raise ValueError("shortconv_kv: single needs one row per sequence")
+    if not u.is_cuda:
+        uf = u[:, :C].float()
+        y = torch.zeros(T, C)
+        cu = cu_q.tolist()
+        for s in range(nseq):
+            a, b = cu[s], cu[s + 1]
+            if b <= a:
+                continue
+            ss = int(sslot[s])
+            p0 = int(pos[a])
+            hist = torch.zeros(taps - 1, C)
+            if ss >= 0 and taps > 1:
+                hist = state[ss].float().clone()
+                for i in range(taps - 1):            # state row i holds position p0 - (taps - 1) + i
+                    if p0 - (taps - 1) + i < 0:
+                        hist[i] = 0
+            ext = torch.cat([hist, uf[a:b]], 0)
+            for j in range(taps):
+                y[a:b] += w[:, j].float() * ext[j:j + (b - a)]
+            if ss >= 0 and taps > 1:
+                state[ss] = ext[-(taps - 1):].to(state.dtype)
+        q = y[:, :Cq].to(u.dtype)
+        k = y[:, Cq:Cq + Ck]
+        v = y[:, Cq + Ck:]
+        if vfirst_out is not None:
+            vfirst_out.copy_(v)
+        if vfirst_in is not None:
+            v = (1.0 - lam.float()) * v + lam.float() * vfirst_in
+        sl = slots.long()
+        ok = sl >= 0
+        blk, off = sl[ok] // BS, sl[ok] % BS
+        k_cache[blk, :, off] = k[ok].view(-1, G, Dk).to(k_cache.dtype)
+        v_cache[blk, :, off] = v[ok].view(-1, G, Dv).to(v_cache.dtype)
+        return q
+    f32 = u.dtype == torch.float32
+    if u.dtype not in (torch.float32, torch.bfloat16) or any(t.dtype != u.dtype for t in (state, k_cache, v_cache)):
+        raise ValueError("shortconv_kv: projection, state and caches share one dtype (bf16 or fp32)")
+    if u.stride(1) != 1 or w.dtype != torch.float32 or not w.is_contiguous() or not state.is_contiguous():
+        raise ValueError("shortconv_kv: bad strides")
+    for t in (row_seq, cu_q, pos, slots, sslot):
+        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+    for t in (vfirst_in, vfirst_out):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (T, Cv))
+    assert (vfirst_in is None) == (lam is None) and (lam is None or lam.dtype == torch.float32)
+    q = torch.empty(T, Cq, dtype=u.dtype, device=u.device)
+    _check(lib().la_shortconv_kv(int(f32), int(single), u.data_ptr(), u.stride(0), w.data_ptr(), taps, Cq, Ck, Cv,
+                                 row_seq.data_ptr(), cu_q.data_ptr(), pos.data_ptr(), slots.data_ptr(),
+                                 sslot.data_ptr(), state.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
+                                 v_cache.data_ptr(), G, Dk, Dv, BS, _ptr(vfirst_in), _ptr(vfirst_out), _ptr(lam), T,
+                                 nseq, _stream()), "la_shortconv_kv")
+    return q
+
+
+def alibi_slopes(H: int, device=None) -> torch.Tensor:
+    """Per-head distance slopes 2^(-8 (h + 1) / H), fp32 [H]."""
+    return torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], dtype=torch.float32, device=device)
+
+
+def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_seq: torch.Tensor, pos: torch.Tensor,
+             block_tables: torch.Tensor, H: int, scale: float, softcap: float = 0.0,
+             slopes: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None, chunk: int = 0,
+             window: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention with reshaped scores over row-major paged K/V ([blocks, G, BS, Dk / Dv]); one
+    query row per token, row r belonging to sequence row_seq[r] (block_tables row) at position
+    pos[r], its keys 0..pos[r] already in the pools.  Per head g: s = scale q.k, softcap tanh,
+    minus slopes[g] * distance; then the heads' scores are mixed by talk [H, H]; keys are visible
+    within the query's chunk of `chunk` positions and the last `window` positions (0: no limit);
+    softmax; values of width Dv; each head's output times sigmoid(gate[r, h]) (gate: [T, H] view,
+    any row stride).  Returns [T, H * Dv] in q's dtype; scores and softmax in fp32."""
+    T = q.shape[0]
+    G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    Dv = v_cache.shape[3]
+    if q.shape[1] != H * Dk or H % G or row_seq.shape[0] != T or pos.shape[0] != T:
+        raise ValueError("attn_mix: operand shapes do not fit")
+    if not q.is_cuda:
+        out = torch.zeros(T, H, Dv)
+        rep = H // G
+        qf = q.float().view(T, H, Dk)
+        for r in range(T):
+            i = int(pos[r])
+            lo = (i // chunk) * chunk if chunk > 0 else 0
+            if window > 0:
+                lo = max(lo, i - window + 1)
+            js = torch.arange(lo, i + 1)
+            tab = block_tables[int(row_seq[r])].long()
+            blk, off = tab[js // BS], js % BS
+            kk = k_cache[blk, :, off].float().repeat_interleave(rep, 1)     # [n, H, Dk]
+            vv = v_cache[blk, :, off].float().repeat_interleave(rep, 1)
+            s = torch.einsum("hd,nhd->hn", qf[r], kk) * scale
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
+            if slopes is not None:
+                s = s - slopes.float().view(H, 1) * (i - js).float().view(1, -1)
+            if talk is not None:
+                s = talk.float() @ s
+            o = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[r].float()).view(H, 1)
+            out[r] = o
+        return out.view(T, H * Dv).to(q.dtype)
+    f32 = q.dtype == torch.float32
+    if q.dtype not in (torch.float32, torch.bfloat16) or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise ValueError("attn_mix: q and the caches share one dtype (bf16 or fp32)")
+    if not (q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and block_tables.is_contiguous()):
+        raise ValueError("attn_mix: operands must be contiguous")
+    for t in (row_seq, pos, block_tables):
+        assert t.dtype == torch.int32 and t.is_cuda
+    for t in (slopes, talk):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    assert slopes is None or slopes.numel() == H
+    assert talk is None or tuple(talk.shape) == (H, H)
+    ldg = 0
+    if gate is not None:
+        if gate.dtype != q.dtype or tuple(gate.shape) != (T, H) or gate.stride(1) != 1:
+            raise ValueError("attn_mix: gate must be a [T, H] view of q's dtype with unit column stride")
+        ldg = gate.stride(0)
+    out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    _check(lib().la_attn_mix_rows(int(f32), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), row_seq.data_ptr(),
+                                  pos.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], T, H, G, Dk, Dv, BS,
+                                  float(scale), float(softcap), _ptr(slopes), _ptr(talk), int(chunk), int(window),
+                                  _ptr(gate), ldg, out.data_ptr(), _stream()), "la_attn_mix_rows")
+    return out
+
+
+def router_sigmoid(xn: torch.Tensor, router: torch.Tensor, corr: Optional[torch.Tensor], topk: int,
+                   renorm: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Sigmoid-score router: s = sigmoid(xn @ router^T) in fp32; the topk experts with the largest
+    s + corr (corr: selection only) are chosen, their weights are s / (sum of the chosen s + 1e-20)
+    (renorm) or s.  Returns (ids [T, topk] int32, weights [T * topk] fp32)."""
+    T, D = xn.shape
+    E = router.shape[0]
+    if not xn.is_cuda:
+        s = torch.sigmoid(xn.float() @ router.float().t())
+        c = s if corr is None else s + corr.float()
+        idx = torch.topk(c, topk, -1).indices
+        w = s.gather(1, idx)
+        if renorm:
+            w = w / (w.sum(-1, keepdim=True) + 1e-20)
+        return idx.to(torch.int32), w.reshape(-1).float()
+    assert xn.dtype in (torch.bfloat16, torch.float32) and xn.stride(1) == 1
+    assert router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == D
+    assert corr is None or (corr.dtype == torch.float32 and corr.numel() == E)
+    ids = torch.empty(T, topk, dtype=torch.int32, device=xn.device)
+    wts = torch.empty(T * topk, dtype=torch.float32, device=xn.device)
+    _check(lib().la_router_sigmoid(int(xn.dtype == torch.float32), xn.data_ptr(), xn.stride(0), router.data_ptr(),
+                                   _ptr(corr), E, D, T, topk, int(renorm), ids.data_ptr(), wts.data_ptr(), _stream()),
+           "la_router_sigmoid")
+    return ids, wts
+
+
+def moe_pairs(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor, ids: torch.Tensor,
+              wts: torch.Tensor) -> torch.Tensor:
+    """Routed gated experts as (token, expert) pair GEMVs on dense stacked weights (small batches,
+    any width, no host sync): y[t] = sum_k wts[t, k] * Wd[e] (silu(Wg[e] x[t]) * (Wu[e] x[t])),
+    e = ids[t, k].  wg / wu [E, F, D], wd [E, D, F] in x's dtype (bf16 or fp32).  Returns fp32 [T, D]."""
+    T, D = x.shape
+    E, F = wg.shape[0], wg.shape[1]
+    topk = ids.shape[1]
+    if not x.is_cuda:
+        xf = x.float()
+        y = torch.zeros(T, D)
+        wv = wts.view(T, topk)
+        for t in range(T):
+            for k in range(topk):
+                e = int(ids[t, k])
+                h = torch.nn.functional.silu(wg[e].float() @ xf[t]) * (wu[e].float() @ xf[t])
+                y[t] += wv[t, k] * (wd[e].float() @ h)
+        return y
+    for w_ in (wg, wu, wd):
+        assert w_.dtype == x.dtype and w_.is_contiguous()
+    assert tuple(wu.shape) == (E, F, D) and tuple(wd.shape) == (E, D, F) and x.is_contiguous()
+    assert ids.dtype == torch.int32 and ids.is_contiguous() and wts.dtype == torch.float32
+    h = torch.empty(T * topk, F, dtype=x.dtype, device=x.device)
+    y = torch.empty(T, D, dtype=torch.float32, device=x.device)
+    _check(lib().la_moe_pairs(int(x.dtype == torch.float32), x.data_ptr(), wg.data_ptr(), wu.data_ptr(), wd.data_ptr(),
+                              ids.data_ptr(), wts.data_ptr(), T, topk, D, F, E, h.data_ptr(), y.data_ptr(), _stream()),
+           "la_moe_pairs")
+    return y
 
 
 # ---------------------------------------------------------------------------------------

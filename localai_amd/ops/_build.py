@@ -28,7 +28,9 @@ def _torch_lib() -> str:
 
 # per-file hipcc flags: the prefill GEMM's dequant runs beside MFMAs, where the packed
 # v_pk_fma_f32 the SLP vectoriser forms issues slower than two scalar FMAs (profiles/r5_prefill_gemm.md)
-FILE_FLAGS = {"gemm_bs.hip": ["-fno-slp-vectorize"]}
+_NO_PK_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]   # scalar fp32 math only
+FILE_FLAGS = {"gemm_bs.hip": ["-fno-slp-vectorize"], "shortconv.hip": _NO_PK_F32, "attention_mix.hip": _NO_PK_F32,
+              "moe_dense.hip": _NO_PK_F32}
 
 
 def _sources():
@@ -62,7 +64,23 @@ def build_variant(name: str, defines, verbose: bool = False, jobs: int = 8) -> P
     return _build_lib(HERE / name, list(defines), False, verbose, jobs)
 
 
-def _build_lib(LIB: Path, defines, force: bool, verbose: bool, jobs: int) -> Path:
+def subset_path(files) -> Path:
+    tag = hashlib.sha256(",".join(sorted(files)).encode()).hexdigest()[:8]
+    return HERE / f"_la_kernels_part_{tag}.so"
+
+
+def build_subset(files, verbose: bool = False, jobs: int = 8) -> Path:
+    """A library of only the named kernel sources (ops/_la_kernels_part_<tag>.so): what one model
+    family launches, for a first run on a checkout where the whole library is not built yet.
+    Entry points of the other sources are absent from it; calling one fails loudly."""
+    names = sorted(set(files))
+    missing = [n for n in names if not (CSRC / n).exists()]
+    if missing:
+        raise FileNotFoundError(f"kernel sources not found: {missing}")
+    return _build_lib(subset_path(names), [], False, verbose, jobs, sources=[CSRC / n for n in names])
+
+
+def _build_lib(LIB: Path, defines, force: bool, verbose: bool, jobs: int, sources=None) -> Path:
     stamp = LIB.with_suffix(".stamp")
     dig = _digest() + ("".join(defines) if defines else "")
     if not force and LIB.exists() and stamp.exists() and stamp.read_text().strip() == dig:
@@ -83,7 +101,7 @@ def _build_lib(LIB: Path, defines, force: bool, verbose: bool, jobs: int) -> Pat
         return obj
 
     with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
-        objs = list(ex.map(compile_one, _sources()))
+        objs = list(ex.map(compile_one, sources if sources is not None else _sources()))
     tl = _torch_lib()
     tmp = LIB.with_suffix(".so.tmp")
     cmd = [_hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs),

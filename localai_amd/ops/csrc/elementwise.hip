@@ -430,6 +430,7 @@ __global__ __launch_bounds__(256) void rope_kv8_kernel(Src qkv, const int* __res
 //               mode 1: GELU(tanh) out[t][i] = gelu(x[t][i])             (src width F)
 //               mode 2: GELU-quick (CLIP)  x * sigmoid(1.702 x)
 //               mode 3: GeGLU (Gemma)  out[t][i] = gelu(x[t][i]) * x[t][F+i]   (src width 2F)
+//               mode 4: squared ReLU  out[t][i] = max(x[t][i], 0)^2           (src width F)
 LA_DEV float gelu_tanh(float x) { return 0.5f * x * (1.f + tanhf(0.7978845608f * (x + 0.044715f * x * x * x))); }
 
 __global__ __launch_bounds__(256) void act_kernel(Src src, bf16* __restrict__ out, int F, int mode) {
@@ -450,6 +451,12 @@ __global__ __launch_bounds__(256) void act_kernel(Src src, bf16* __restrict__ ou
     for (int j = 0; j < 4; ++j) {
       const float x = a[j];
       o[j] = 0.5f * x * (1.f + tanhf(0.7978845608f * (x + 0.044715f * x * x * x)));
+    }
+  } else if (mode == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float x = fmaxf(a[j], 0.f);
+      o[j] = x * x;
     }
   } else {
 #pragma unroll
@@ -483,6 +490,12 @@ __global__ __launch_bounds__(256) void act8_kernel(const bf16* __restrict__ src,
     for (int j = 0; j < 8; ++j) {
       const float x = (float)a[j];
       ob[j] = (bf16)(0.5f * x * (1.f + tanhf(0.7978845608f * (x + 0.044715f * x * x * x))));
+    }
+  } else if (mode == 4) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float x = fmaxf((float)a[j], 0.f);
+      ob[j] = (bf16)(x * x);
     }
   } else {
 #pragma unroll
@@ -654,7 +667,7 @@ extern "C" int la_rope_kv(const void* qkv_p, long slab, int S, const void* bias,
 
 extern "C" int la_act(const void* p, long slab, int S, const void* bias, void* out, int T, int F, int mode,
                       void* stream) {
-  if ((F & 3) || mode < 0 || mode > 3) return -1;
+  if ((F & 3) || mode < 0 || mode > 4) return -1;
   if (S == 0 && bias == nullptr && (F & 7) == 0 && ((uintptr_t)p & 15) == 0 && ((uintptr_t)out & 15) == 0) {
     dim3 grid((F / 8 + 255) / 256, T);
     hipLaunchKernelGGL(la::act8_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)p, (bf16*)out, F,

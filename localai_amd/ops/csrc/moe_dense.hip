@@ -1,0 +1,142 @@
+// Mixture-of-experts pieces for dense (bf16 / fp32) expert weights of any width:
+//   * a router with sigmoid scores, an optional selection-only correction and normalised weights;
+//   * the routed experts of small batches as (token, expert) pair GEMVs: gate|up with the SiLU
+//     gating fused, then the down projection with the weighted top-k combine fused, no atomics.
+// Larger batches group rows by expert and run library GEMMs (the caller's choice).
+#include "common.h"
+
+namespace la {
+
+// One wave per token: z_e = router[e] . x (fp32), s = sigmoid(z); the `topk` largest s + corr are
+// chosen (ties: lowest expert id), their weights are s / (sum of the chosen s + 1e-20).
+template <typename AT>
+__global__ __launch_bounds__(256) void router_sigmoid_kernel(const AT* __restrict__ x, long ldx,
+                                                             const float* __restrict__ router,
+                                                             const float* __restrict__ corr, int E, int D, int T,
+                                                             int topk, int renorm, int* __restrict__ ids,
+                                                             float* __restrict__ wts) {
+  __shared__ float sc[4][256];
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + w;
+  const bool live = t < T;
+  const AT* xr = x + (long)(live ? t : 0) * ldx;
+  for (int e = 0; e < E; ++e) {
+    float a = 0.f;
+    for (int d = lane; d < D; d += 64) a = fmaf(router[(long)e * D + d], (float)xr[d], a);
+    a = wave_sum(a);
+    if (lane == 0) sc[w][e] = 1.f / (1.f + __expf(-a));
+  }
+  __syncthreads();
+  float sum = 0.f, my_s = 0.f;
+  int my_id = 0;
+  uint32_t taken = 0;   // bit i: this lane's expert e = lane + 64 * i is already chosen
+  for (int k = 0; k < topk; ++k) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = 0; i < 4; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && !((taken >> i) & 1u)) {
+        const float c = sc[w][e] + (corr ? corr[e] : 0.f);
+        if (c > best || (c == best && e < bi)) { best = c; bi = e; }
+      }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+    const float s = sc[w][bi];
+    sum += s;
+    if (lane == k) { my_s = s; my_id = bi; }
+  }
+  if (live && lane < topk) {
+    ids[(long)t * topk + lane] = my_id;
+    wts[(long)t * topk + lane] = renorm ? my_s / (sum + 1e-20f) : my_s;
+  }
+}
+
+// h[p][f] = silu(Wg[e_p][f] . x[t_p]) * (Wu[e_p][f] . x[t_p]),  p = t * topk + slot; a wave per (p, f)
+template <typename AT, typename WT>
+__global__ __launch_bounds__(256) void moe_pair_glu_kernel(const AT* __restrict__ x, const WT* __restrict__ wg,
+                                                           const WT* __restrict__ wu, const int* __restrict__ ids,
+                                                           int topk, int D, int F, int E, AT* __restrict__ h) {
+  const int p = blockIdx.y;
+  const int f = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (f >= F) return;
+  const int e = ids[p];
+  if (e < 0 || e >= E) { if (lane == 0) h[(long)p * F + f] = (AT)0.f; return; }
+  const AT* xr = x + (long)(p / topk) * D;
+  const WT* g = wg + ((long)e * F + f) * D;
+  const WT* u = wu + ((long)e * F + f) * D;
+  float a = 0.f, b = 0.f;
+  for (int d = lane; d < D; d += 64) {
+    const float xv = (float)xr[d];
+    a = fmaf((float)g[d], xv, a);
+    b = fmaf((float)u[d], xv, b);
+  }
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if (lane == 0) h[(long)p * F + f] = (AT)(silu(a) * b);
+}
+
+// y[t][d] = sum_slot w[p] * (Wd[e_p][d] . h[p]); a wave per (t, d), slots in order (deterministic)
+template <typename AT, typename WT>
+__global__ __launch_bounds__(256) void moe_pair_down_kernel(const AT* __restrict__ h, const WT* __restrict__ wd,
+                                                            const int* __restrict__ ids, const float* __restrict__ wts,
+                                                            int topk, int D, int F, int E, float* __restrict__ y) {
+  const int t = blockIdx.y;
+  const int d = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (d >= D) return;
+  float acc = 0.f;
+  for (int k = 0; k < topk; ++k) {
+    const int p = t * topk + k, e = ids[p];
+    if (e < 0 || e >= E) continue;
+    const WT* wr = wd + ((long)e * D + d) * F;
+    const AT* hr = h + (long)p * F;
+    float a = 0.f;
+    for (int f = lane; f < F; f += 64) a = fmaf((float)wr[f], (float)hr[f], a);
+    acc = fmaf(wts[p], wave_sum(a), acc);
+  }
+  if (lane == 0) y[(long)t * D + d] = acc;
+}
+
+}  // namespace la
+
+extern "C" int la_router_sigmoid(int f32, const void* x, long ldx, const void* router, const void* corr, int E, int D,
+                                 int T, int topk, int renorm, void* ids, void* wts, void* stream) {
+  using namespace la;
+  if (E < 1 || E > 256 || topk < 1 || topk > E || topk > 64 || T <= 0) return -1;
+  dim3 grid((T + 3) / 4);
+  if (f32)
+    hipLaunchKernelGGL((router_sigmoid_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, ldx,
+                       (const float*)router, (const float*)corr, E, D, T, topk, renorm, (int*)ids, (float*)wts);
+  else
+    hipLaunchKernelGGL((router_sigmoid_kernel<bf16>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, ldx,
+                       (const float*)router, (const float*)corr, E, D, T, topk, renorm, (int*)ids, (float*)wts);
+  return (int)hipGetLastError();
+}
+
+// f32: activations and weights fp32 (else both bf16).  x [T, D], wg / wu [E, F, D], wd [E, D, F],
+// ids [T * topk], wts [T * topk] -> h [T * topk, F] (scratch, activation type), y [T, D] fp32.
+extern "C" int la_moe_pairs(int f32, const void* x, const void* wg, const void* wu, const void* wd, const void* ids,
+                            const void* wts, int T, int topk, int D, int F, int E, void* h, void* y, void* stream) {
+  using namespace la;
+  if (T <= 0 || topk < 1 || D < 1 || F < 1) return -1;
+  const int P = T * topk;
+  if (P > 65535 || T > 65535) return -2;
+  dim3 g1((F + 3) / 4, P), g2((D + 3) / 4, T);
+  hipStream_t s = (hipStream_t)stream;
+  if (f32) {
+    hipLaunchKernelGGL((moe_pair_glu_kernel<float, float>), g1, dim3(256), 0, s, (const float*)x, (const float*)wg,
+                       (const float*)wu, (const int*)ids, topk, D, F, E, (float*)h);
+    hipLaunchKernelGGL((moe_pair_down_kernel<float, float>), g2, dim3(256), 0, s, (const float*)h, (const float*)wd,
+                       (const int*)ids, (const float*)wts, topk, D, F, E, (float*)y);
+  } else {
+    hipLaunchKernelGGL((moe_pair_glu_kernel<bf16, bf16>), g1, dim3(256), 0, s, (const bf16*)x, (const bf16*)wg,
+                       (const bf16*)wu, (const int*)ids, topk, D, F, E, (bf16*)h);
+    hipLaunchKernelGGL((moe_pair_down_kernel<bf16, bf16>), g2, dim3(256), 0, s, (const bf16*)h, (const bf16*)wd,
+                       (const int*)ids, (const float*)wts, topk, D, F, E, (float*)y);
+  }
+  return (int)hipGetLastError();
+}

@@ -223,7 +223,10 @@ class Tokenizer:
             hit = c.get((s, at_start))
             if hit is not None:
                 return list(hit)
-        if self.model == "gpt2":
+        if self.model == "numeric":
+            # checkpoints without a vocabulary: the text IS token ids ("12 7 <3>" -> [12, 7, 3])
+            ids = [int(m) for m in re.findall(r"\d+", s) if int(m) < len(self.tokens)]
+        elif self.model == "gpt2":
             if getattr(self, "_pre_re", None) is not None:
                 ids = self._bpe_fast(s)
             else:
