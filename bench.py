@@ -76,6 +76,10 @@ def parse():
                     help="ranks: every rank serves its own gateway + load (summed); gateway: rank 0's ONE "
                          "gateway serves all N GPUs (data_parallel_size: N behind parallel/replicas.py), the "
                          "other ranks' engines answer it over backend.proto gRPC")
+    ap.add_argument("--design-compare", default="",
+                    help="instead of the headline workload: prefill and decode tokens/s of a model design "
+                         "(suganex) beside the closest decoder family at equal layer sizes, random weights, one GPU")
+    ap.add_argument("--design-sizes", default="2k,4k", help="--design-compare: layer sizes (2k, 4k)")
     ap.add_argument("--n-draft", type=int, default=0,
                     help="engine mode: n-gram speculative draft length (model-config n_draft); 0 = off")
     return ap.parse_args()
@@ -121,6 +125,10 @@ def spawn_ranks(args) -> int:
 
 def main():
     args = parse()
+    if args.design_compare:
+        from localai_amd.utils import design_bench
+        design_bench.run(args.design_compare, args.design_sizes.split(","), args.cache_dir, iters=max(1, args.steps))
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(spawn_ranks(args))
     loadgen = None

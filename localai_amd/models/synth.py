@@ -1304,3 +1304,53 @@ def write_piper_voice(path: str, seed: int = 0, sampling_rate: int = 8000):
     with open(path + ".json", "w", encoding="utf-8") as f:
         json.dump(conf, f, ensure_ascii=False)
     return m
+
+
+def write_suganex(out_dir: str, width: int = 256, n_layer: int = 2, heads: int = 4, kv_heads: int = 2, dim: int = 64,
+                  vdim: int = 64, conv: int = 4, chunk: int = 256, ff: int = 1024, experts: int = 0, top: int = 2,
+                  expert_ff: int = 0, vocab: int = 32000, softcap: float = 30.0, seed: int = 0) -> str:
+    """Random-init Suganex checkpoint directory (config.json + model.safetensors, bf16): `n_layer`
+    equal layers, dense feed-forwards of width `ff`, or -- with `experts` -- routed experts of width
+    `expert_ff` (default ff).  Benchmarks and smoke runs; the weights mean nothing."""
+    import json
+
+    import torch
+    from safetensors.torch import save_file
+    os.makedirs(out_dir, exist_ok=True)
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(*shape, s):
+        return (torch.randn(*shape, generator=g, dtype=torch.float32) * s).to(torch.bfloat16)
+
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv, "scale": dim ** -0.5,
+             "softcap": softcap, "v_mix": True, "mask": {"size": chunk}}
+    if experts:
+        mlp = {"kind": "moe", "expert": {"ff": expert_ff or ff}, "router": {"experts": experts, "top": top}}
+    else:
+        mlp = {"kind": "dense", "ff": ff}
+    cfg = {"architecture": "Suganex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+           "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp} for _ in range(n_layer)]}
+    D = width
+    W = {"embed": rnd(vocab, D, s=1.0), "final.norm": rnd(D, s=0.05), "head": rnd(vocab, D, s=D ** -0.5)}
+    for i in range(n_layer):
+        p = f"l{i}."
+        W[p + "norm1"], W[p + "norm2"] = rnd(D, s=0.05), rnd(D, s=0.05)
+        W[p + "mix.q"], W[p + "mix.k"] = rnd(heads * dim, D, s=D ** -0.5), rnd(kv_heads * dim, D, s=D ** -0.5)
+        W[p + "mix.v"], W[p + "mix.g"] = rnd(kv_heads * vdim, D, s=D ** -0.5), rnd(heads, D, s=D ** -0.5)
+        for n, c in (("q", heads * dim), ("k", kv_heads * dim), ("v", kv_heads * vdim)):
+            W[p + f"mix.{n}.conv"] = rnd(c, conv, s=conv ** -0.5)
+        W[p + "mix.vmix"] = torch.tensor(0.25).to(torch.bfloat16)
+        W[p + "mix.talk"] = (torch.eye(heads) + 0.1 * torch.randn(heads, heads, generator=g)).to(torch.bfloat16)
+        W[p + "mix.o"] = rnd(D, heads * vdim, s=(heads * vdim) ** -0.5)
+        if experts:
+            F = expert_ff or ff
+            W[p + "mlp.router"], W[p + "mlp.correction"] = rnd(experts, D, s=D ** -0.5), rnd(experts, s=0.1)
+            for e in range(experts):
+                W[p + f"mlp.e{e}.gate"], W[p + f"mlp.e{e}.up"] = rnd(F, D, s=D ** -0.5), rnd(F, D, s=D ** -0.5)
+                W[p + f"mlp.e{e}.down"] = rnd(D, F, s=F ** -0.5)
+        else:
+            W[p + "mlp.up"], W[p + "mlp.down"] = rnd(ff, D, s=D ** -0.5), rnd(D, ff, s=ff ** -0.5)
+    with open(os.path.join(out_dir, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file(W, os.path.join(out_dir, "model.safetensors"))
+    return out_dir

@@ -1,0 +1,155 @@
+"""Prefill and decode throughput of a model design beside the closest decoder family at equal
+layer sizes (bench.py --design-compare): random weights, bf16, one GPU.
+
+For each size two pairs of two-layer models are built -- dense feed-forwards (Suganex vs a llama
+checkpoint) and routed experts (Suganex vs a Mixtral-style checkpoint), both stored as dense bf16
+weights so every GEMM takes the same library path -- and each is timed through its engine's own
+batch construction (native scheduler, paged KV pool, state slots) and `model.forward`:
+  prefill: `n_seq` prompts of `prompt` tokens in one batch, tokens/s;
+  decode:  `batch` sequences holding `context` tokens each, one token per sequence and step, tokens/s.
+The forward is repeated on the same batch (it rewrites the same K/V slots), so the numbers are the
+kernels' and the GEMMs', without the host's planning time.
+"""
+from __future__ import annotations
+
+import json
+import os
+import time
+from typing import Dict, List
+
+import numpy as np
+import torch
+
+SIZES = {
+    # name: width, heads, kv heads, head width, dense ff, experts, top, expert ff, chunk
+    "2k": dict(width=2048, heads=16, kv=4, dim=128, ff=8192, experts=8, top=2, eff=2048, chunk=1024),
+    "tiny": dict(width=256, heads=4, kv=2, dim=64, ff=512, experts=4, top=2, eff=256, chunk=64),   # dry runs
+    "4k": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, experts=8, top=2, eff=3584, chunk=1024),
+}
+VOCAB = 32000
+
+
+def _models(size: str, cache: str) -> Dict[str, str]:
+    from ..models import synth
+    s = SIZES[size]
+    out = {}
+    for kind in ("dense", "moe"):
+        moe = kind == "moe"
+        p = os.path.join(cache, f"suganex-{size}-{kind}")
+        if not os.path.exists(os.path.join(p, "model.safetensors")):
+            synth.write_suganex(p, width=s["width"], n_layer=2, heads=s["heads"], kv_heads=s["kv"], dim=s["dim"],
+                                vdim=s["dim"], conv=4, chunk=s["chunk"], ff=s["ff"], experts=s["experts"] if moe else 0,
+                                top=s["top"], expert_ff=s["eff"], vocab=VOCAB)
+        out[f"suganex-{kind}"] = p
+        g = os.path.join(cache, f"llama-{size}-{kind}-f16.gguf")
+        if not os.path.exists(g):
+            pre = synth.Preset(n_layer=2, n_embd=s["width"], n_head=s["heads"], n_head_kv=s["kv"], head_dim=s["dim"],
+                               n_ff=s["eff"] if moe else s["ff"], n_vocab=VOCAB, ctx=8192, qtype="F16",
+                               n_expert=s["experts"] if moe else 0, n_expert_used=s["top"] if moe else 0,
+                               tokenizer="mistral", name=f"llama-{size}-{kind}")
+            synth.write_model(g + ".partial", pre)
+            os.replace(g + ".partial", g)
+        out[("mixtral" if moe else "llama") + f"-{kind}"] = g
+    return out
+
+
+def DEVICE() -> str:
+    return "cuda:0" if torch.cuda.is_available() else "cpu"
+
+
+def _time(fn, iters: int) -> float:
+    for _ in range(2):
+        fn()
+    if not torch.cuda.is_available():
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        return (time.perf_counter() - t0) / iters
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / 1e3 / iters
+
+
+def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters: int) -> Dict[str, float]:
+    from .. import ops
+    from ..engine.llm_engine import EngineConfig, LLMEngine
+    from ..models.decoder import DecoderModel, ForwardBatch
+    tokens = max(n_seq * prompt, batch * (context + 32))
+    eng = LLMEngine(EngineConfig(model_path=path, device=DEVICE(), context_size=max(prompt, context + 32) + 32,
+                                 max_num_seqs=max(n_seq, batch), max_batched_tokens=n_seq * prompt, block_size=32,
+                                 max_kv_tokens=tokens + 64 * max(n_seq, batch), prefix_cache=False, use_graphs=False,
+                                 blas_tune=False))
+    rng = np.random.default_rng(0)
+    dm = isinstance(eng.model, DecoderModel)
+
+    def batch_of(ids, n):
+        for i in ids:
+            if eng.sched.has(i):
+                eng.sched.extend(i, rng.integers(0, VOCAB, size=n).tolist())
+            else:
+                eng.sched.add(i, rng.integers(0, VOCAB, size=n).tolist(), 0)
+        plan = eng.sched.schedule_explicit([(i, n) for i in ids])
+        k, q = len(ids), plan["p_qlen"]
+        dec = bool(plan["p_decode"].all()) and n == 1
+        fb = ForwardBatch(tokens=eng._dev(plan["p_tokens"]), pos=eng._dev(plan["p_pos"]), slots=eng._dev(plan["p_slots"]),
+                          decode=dec and dm, block_tables=eng._dev(plan["p_bt"]),
+                          logits_idx=eng._dev(np.asarray(plan["p_cu"][1:] - 1, dtype=np.int64)))
+        if dec and dm:
+            fb.seq_lens, fb.max_len = eng._dev(plan["p_ctx"]), int(plan["p_ctx"].max())
+        else:
+            fb.cu_q, fb.ctx_lens = eng._dev(plan["p_cu"]), eng._dev(plan["p_ctx"])
+            if dm:
+                fb.tiles = ops.prefill_tiles(q.tolist(), eng.device)
+        if not dm:
+            fb.sslots = eng._dev(plan["p_sslot"])
+            fb.row_seq = eng._dev(np.repeat(np.arange(k, dtype=np.int32), q))
+        return fb
+
+    out = {}
+    fb = batch_of(list(range(1, n_seq + 1)), prompt)
+    t = _time(lambda: eng.model.forward(fb, eng.kv), iters)
+    out["prefill_tok_s"] = n_seq * prompt / t
+    out["prefill_ms"] = t * 1e3
+    for i in range(1, n_seq + 1):
+        eng.sched.finish(i)
+    ids = list(range(100, 100 + batch))
+    left = context
+    while left > 0:   # fill the contexts in chunks that fit one batch
+        n = min(left, max(1, (n_seq * prompt) // batch))
+        eng.model.forward(batch_of(ids, n), eng.kv)
+        left -= n
+    fb = batch_of(ids, 1)
+    t = _time(lambda: eng.model.forward(fb, eng.kv), iters * 4)
+    out["decode_tok_s"] = batch / t
+    out["decode_ms"] = t * 1e3
+    del eng
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+    return out
+
+
+def run(design: str, sizes: List[str], cache: str, n_seq: int = 4, prompt: int = 2048, batch: int = 64,
+        context: int = 1024, iters: int = 5) -> dict:
+    if design != "suganex":
+        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex)")
+    os.makedirs(cache, exist_ok=True)
+    res = {"design": design, "dtype": "bf16", "data": "synthetic", "layers": 2,
+           "workload": {"prefill": f"{n_seq} x {prompt} tokens", "decode": f"batch {batch} at context {context}"},
+           "sizes": {}}
+    for size in sizes:
+        t0 = time.time()
+        paths = _models(size, cache)
+        row = {}
+        for name, p in paths.items():
+            row[name] = {k: round(v, 3 if k.endswith("ms") else 1)
+                         for k, v in _measure(p, n_seq, prompt, batch, context, iters).items()}
+            print(f"# {size} {name}: {row[name]}", flush=True)
+        res["sizes"][size] = dict(SIZES[size], **row)
+        print(f"# {size} done in {time.time() - t0:.0f} s", flush=True)
+    print(json.dumps(res), flush=True)
+    return res
