@@ -925,6 +925,8 @@ class LLMEngine:
                               cu_q=self._dev(cu), ctx_lens=self._dev(plan["p_ctx"]), logits_idx=idx(rows),
                               sslots=self._dev(plan["p_sslot"]),
                               row_seq=self._dev(np.repeat(np.arange(n, dtype=np.int32), qlens)))
+            # the leading portions on the tile kernel, the single-token rows after them on the row kernel
+            fb.tiles, fb.tile_rows = self.model.prefill_tiles(qlens[:nc], self.device) if nc else (None, 0)
             if not rows:
                 self.model.forward(fb, self.kv)
                 return None
@@ -937,9 +939,8 @@ class LLMEngine:
             fb = ForwardBatch(tokens=self._dev(plan["p_tokens"][:tp]), pos=self._dev(plan["p_pos"][:tp]),
                               slots=self._dev(plan["p_slots"][:tp]), decode=False,
                               block_tables=self._dev(plan["p_bt"][:nc]), cu_q=self._dev(cu[:nc + 1]),
-                              ctx_lens=self._dev(plan["p_ctx"][:nc]),
-                              tiles=ops.prefill_tiles(qlens[:nc].tolist(), self.device) if gpu else None,
-                              logits_idx=idx(prow))
+                              ctx_lens=self._dev(plan["p_ctx"][:nc]), logits_idx=idx(prow))
+            fb.tiles, fb.tile_rows = self.model.prefill_tiles(qlens[:nc], self.device)
             if prow:
                 lg = self.model.forward(fb, self.kv).float()
                 out.update({r: lg[k] for k, r in enumerate(prow)})
@@ -989,10 +990,9 @@ class LLMEngine:
         fb = ForwardBatch(
             tokens=self._dev(tokens), pos=self._dev(plan["p_pos"]), slots=self._dev(plan["p_slots"]),
             decode=False, block_tables=self._dev(plan["p_bt"]), cu_q=self._dev(cu), ctx_lens=self._dev(plan["p_ctx"]),
-            tiles=(ops.prefill_tiles(qlens.tolist(), self.device)
-                   if self.device.type == "cuda" and isinstance(self.model, DecoderModel) else None),
             logits_idx=self._dev(np.array(rows, dtype=np.int64)) if rows else None,
             inject_idx=inj_idx, inject_rows=inj_rows)
+        fb.tiles, fb.tile_rows = self.model.prefill_tiles(qlens, self.device)
         if self.stateful:
             fb.sslots = self._dev(plan["p_sslot"])
             fb.row_seq = self._dev(np.repeat(np.arange(len(ids), dtype=np.int32), qlens))

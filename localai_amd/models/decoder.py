@@ -217,6 +217,7 @@ class ForwardBatch:
     cu_q: Optional[torch.Tensor] = None       # prefill: [nseq+1] i32
     ctx_lens: Optional[torch.Tensor] = None   # prefill: [nseq] i32
     tiles: Optional[torch.Tensor] = None      # prefill: attention work tiles
+    tile_rows: int = 0                        # rows the tiles cover (mixed batches: the leading portions)
     logits_idx: Optional[torch.Tensor] = None  # rows to project to logits (None: all)
     inject_idx: Optional[torch.Tensor] = None  # prefill rows whose embedding is given (images)
     inject_rows: Optional[torch.Tensor] = None  # [n, n_embd] f32
@@ -253,15 +254,17 @@ class KVCache:
     def layered(cls, specs, num_blocks: int, block_size: int, device, dtype=torch.bfloat16,
                 state_slots: int = 0) -> "KVCache":
         """Pools for layers that differ in shape: specs[i] = (kv heads, key width, value width,
-        state shape or None).  K and V pages are both row-major [num_blocks, heads, block_size,
-        width] (ops.kv_pages: the layout ops.shortconv_kv writes and ops.attn_mix reads); layers
+        state shape or None).  K pages are row-major [num_blocks, heads, block_size, width]
+        (ops.kv_pages), V pages transposed per 8 keys like the other families' (ops.v_pages); layers
         with a state shape get a pool [state_slots, *shape] beside them, indexed by the scheduler's
         state slots.  Slots are never cleared: a kernel reads of a slot only what lies at
         positions >= 0 of the sequence that holds it."""
         kv = cls.__new__(cls)
         kv.num_blocks, kv.block_size = num_blocks, block_size
         kv.k = [ops.kv_pages(num_blocks, g, block_size, dk, dtype, device) for g, dk, _, _ in specs]
-        kv.v = [ops.kv_pages(num_blocks, g, block_size, dv, dtype, device) for g, _, dv, _ in specs]
+        if block_size % 8:
+            raise ValueError(f"block_size {block_size} must be a multiple of 8")
+        kv.v = [ops.v_pages(num_blocks, g, block_size, dv, dtype, device) for g, _, dv, _ in specs]
         kv.state_slots = state_slots
         kv.state = None
         if state_slots > 0:
@@ -582,6 +585,12 @@ class DecoderModel:
 
     def kv_bytes_per_token(self) -> int:
         return 2 * self.hp.n_layer * self.Hkv * self.Dh * 2
+
+    def prefill_tiles(self, q_lens, device):
+        """(attention work tiles of a batch of prompt portions, rows they cover)."""
+        if device.type != "cuda":
+            return None, 0
+        return ops.prefill_tiles([int(n) for n in q_lens], device), int(sum(int(n) for n in q_lens))
 
     def decode_workspace(self, Bp: int, ctx: int, block_size: int):
         return ops.decode_workspace(Bp, self.Hq, self.Hkv, self.Dh, ctx, self.device, block_size)

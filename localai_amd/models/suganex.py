@@ -139,7 +139,7 @@ class _Layer:
 class SuganexModel:
     # what this family launches from ops/csrc (ops.require_kernels: a first run compiles only these)
     kernel_sources = ("elementwise.hip", "shortconv.hip", "attention_mix.hip", "moe_dense.hip", "moe.hip",
-                      "sampling.hip", "decode_loop.hip")
+                      "sampling.hip", "decode_loop.hip", "gemm_skinny.hip")
     stateful = True         # per-sequence convolution tails: state slots, no prefix-cache reuse
     mixed_batches = True    # prompt portions and decode rows of different sequences in one forward
 
@@ -229,6 +229,12 @@ class SuganexModel:
 
     def decode_workspace(self, Bp: int, ctx: int, block_size: int):
         return None
+
+    def prefill_tiles(self, q_lens, device):
+        """(16-row work tiles of the leading prompt portions for ops.attn_mix, rows they cover)."""
+        if device.type != "cuda" or self.f32:
+            return None, 0
+        return ops.attn_mix_tiles(q_lens, device)
 
     def _single_rows(self, T: int):
         a = self._aranges.get(T)
@@ -327,7 +333,8 @@ class SuganexModel:
             q = ops.shortconv_kv(proj, L.conv, m.Cq, m.Ck, m.Cv, row_seq, cu_q, fb.pos, fb.slots, fb.sslots,
                                  kv.state[i], kv.k[i], kv.v[i], vfirst_in=vin, vfirst_out=vout, lam=lam, single=single)
             a = ops.attn_mix(q, kv.k[i], kv.v[i], row_seq, fb.pos, fb.block_tables, m.heads, m.scale, m.softcap,
-                             L.slopes, L.talk, m.chunk, m.window, gate=proj[:, C:C + m.heads])
+                             L.slopes, L.talk, m.chunk, m.window, gate=proj[:, C:C + m.heads],
+                             tiles=None if fb.decode else fb.tiles, tile_rows=fb.tile_rows, cu_q=cu_q)
             o = ops.linear(a, L.wo)
             nxt = self.layers[i + 1].norm1 if i + 1 < n else self.out_norm
             if f is not None:

@@ -121,6 +121,7 @@ def lib():
             "la_decode_advance": [P, P, P, P, P, P, I, I, I, P, I, P, P, P],
             "la_shortconv_kv": [I, I, P, I, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, P, P, P, I, I, P],
             "la_attn_mix_rows": [I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
+            "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
             "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
             "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
@@ -155,6 +156,12 @@ def lib():
             _check(L.la_dec_one_part(int(os.environ["LOCALAI_AMD_DEC_ONE_PART"])), "la_dec_one_part")
         _LIB = L
         return L
+
+
+def _has(name: str) -> bool:
+    """Is the entry point in the loaded library (a partial library, require_kernels, lacks the GEMM
+    families its model does not launch: those shapes take the library GEMM instead)."""
+    return hasattr(lib(), name)
 
 
 def hip_available() -> bool:
@@ -959,7 +966,7 @@ def _autotune_mid(x, ws, key, Ntot):
     cands = []
     if all(w.tile_ok for w in ws):
         tiles = (6, 1, 7, 8, 12) if M > 128 else (7, 12, 14, 3)
-        for t in tiles:
+        for t in tiles if _has("la_qgemm_tile") else ():
             g = _tile_grid(M, N, t)
             base = max(1, round(256 / g))
             # split-K <= 8: every split costs its consumer another fp32 [M, N] slab read
@@ -967,13 +974,13 @@ def _autotune_mid(x, ws, key, Ntot):
                 if S <= min(8, K // 256) and _tile_split_ok(K, S):
                     cands.append(("tile", S, t))
         for v in ((9, 8, 4, 6, 0) if M > 128 else (9, 8, 7, 3)):
-            if not q32_ok(ws, v):
+            if not q32_ok(ws, v) or not _has("la_qgemm32"):
                 continue
             base = max(1, round(256 / _q32_grid(M, N, v)))
             for S in sorted({1, max(1, base // 2), base, base * 2}):
                 if S <= min(8, K // 256) and _tile_split_ok(K, S):
                     cands.append(("q32", S, v))
-    if bs_ok(ws) and (len(ws) == 1 or (len(ws) == 2 and (ws[0].fmt, ws[1].fmt) in _TILE2_PAIRS)):
+    if bs_ok(ws) and _has("la_bsgemm") and (len(ws) == 1 or (len(ws) == 2 and (ws[0].fmt, ws[1].fmt) in _TILE2_PAIRS)):
         for v in ((0, 1, 3) if M > 128 else (1,)):
             base = max(1, round(256 / _bs_grid(M, N, v)))
             for S in sorted({1, max(1, base // 2), base, base * 2}):
@@ -1040,9 +1047,9 @@ def linear_multi(x: torch.Tensor, ws: Sequence[QWeight], bias: Optional[torch.Te
         raise ValueError("linear: x must be contiguous bf16")
     if any(w.fmt == FMT_F32 for w in ws):
         raise ValueError("linear: fp32 weights take fp32 activations")
-    skinny_ok = all(w.K % 256 == 0 for w in ws)
+    skinny_ok = all(w.K % 256 == 0 for w in ws) and _has("la_qgemm_skinny")
     use_skinny = (M <= SKINNY_MAX_M and skinny_ok) if force is None else force == "skinny"
-    tile_ok = TILE_GEMM and all(w.tile_ok for w in ws)
+    tile_ok = TILE_GEMM and all(w.tile_ok for w in ws) and (_has("la_qgemm_tile") or _has("la_qgemm32") or _has("la_bsgemm"))
     S, tile, kind = 0, 0, None
     if force is not None and (force.startswith("q32:") or force.startswith("bs:")):
         kind, v, s_ = force.split(":")
@@ -1059,7 +1066,7 @@ def linear_multi(x: torch.Tensor, ws: Sequence[QWeight], bias: Optional[torch.Te
         choice = _GEMM_CHOICE.get(key)
         if choice is None and GEMM_AUTOTUNE and not torch.cuda.is_current_stream_capturing():
             choice = _autotune_mid(x, ws, key, Ntot)
-        if choice is None and tile_ok:
+        if choice is None and tile_ok and _has("la_qgemm_tile"):
             t, s_ = pick_tile(M, [w.N for w in ws], K)
             choice = ("tile", s_, t)
         if choice is not None and choice[0] in ("tile", "q32", "bs"):
@@ -1718,7 +1725,8 @@ def _attn_ref_prefill(q, kc, vc, cu_q, ctx_lens, bt, scale, softcap=0.0, window=
 # ---------------------------------------------------------------------------------------
 
 def kv_pages(nblk: int, G: int, BS: int, D: int, dtype=torch.bfloat16, device=None) -> torch.Tensor:
-    """Row-major K or V pages [blocks, G, BS, D] (the layout shortconv_kv writes and attn_mix reads)."""
+    """Row-major K pages [blocks, G, BS, D] of any dtype (shortconv_kv writes them, attn_mix reads
+    them; their V pages are v_pages)."""
     return torch.zeros(nblk, G, BS, D, dtype=dtype, device=device)
 
 
@@ -1732,7 +1740,8 @@ def shortconv_kv(u: torch.Tensor, w: torch.Tensor, Cq: int, Ck: int, Cv: int, ro
     (row_seq [T] -> sequence, cu_q [nseq + 1] row ranges, pos [T] positions).  What precedes a
     portion comes from state[sslot[seq]] ([slots, taps - 1, C]: the last taps - 1 projected rows),
     zeros before position 0; the state then advances to the end of the portion.  Returns q [T, Cq];
-    k and v go to the paged pools ([blocks, G, BS, Dk / Dv]) at `slots` (-1: nowhere), v first mixed
+    k and v go to the paged pools (K: kv_pages [blocks, G, BS, Dk]; V: v_pages, transposed per 8 keys,
+    [blocks, G, BS / 8, Dv, 8]) at `slots` (-1: nowhere), v first mixed
     as (1 - lam) v + lam vfirst_in when given; vfirst_out receives the unmixed v (fp32 [T, Cv]).
     single: every sequence brings one row (decode batches): one fused launch."""
     T = u.shape[0]
@@ -1741,6 +1750,8 @@ def shortconv_kv(u: torch.Tensor, w: torch.Tensor, Cq: int, Ck: int, Cv: int, ro
     nseq = cu_q.shape[0] - 1
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     Dv = v_cache.shape[3]
+    if v_cache.dim() != 5 or v_cache.shape[2] * 8 != BS or v_cache.shape[4] != 8:
+        raise ValueError("shortconv_kv: V pages must be [blocks, G, BS / 8, Dv, 8]")
     if (w.shape[0] != C or u.shape[1] < C or Ck != G * Dk or Cv != G * Dv or state.shape[1:] != (max(taps - 1, 0), C)
             or row_seq.shape[0] != T or pos.shape[0] != T or slots.shape[0] != T or sslot.shape[0] != nseq):
         raise ValueError("shortconv_kv: operand shapes do not fit")
@@ -1778,7 +1789,7 @@ def shortconv_kv(u: torch.Tensor, w: torch.Tensor, Cq: int, Ck: int, Cv: int, ro
         ok = sl >= 0
         blk, off = sl[ok] // BS, sl[ok] % BS
         k_cache[blk, :, off] = k[ok].view(-1, G, Dk).to(k_cache.dtype)
-        v_cache[blk, :, off] = v[ok].view(-1, G, Dv).to(v_cache.dtype)
+        v_cache[blk, :, off // 8, :, off % 8] = v[ok].view(-1, G, Dv).to(v_cache.dtype)
         return q
     f32 = u.dtype == torch.float32
     if u.dtype not in (torch.float32, torch.bfloat16) or any(t.dtype != u.dtype for t in (state, k_cache, v_cache)):
@@ -1804,20 +1815,40 @@ def alibi_slopes(H: int, device=None) -> torch.Tensor:
     return torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], dtype=torch.float32, device=device)
 
 
+ATTN_MIX_QT = 16   # query rows per tile of the matrix-core kernel
+ATTN_MIX_TILES = os.environ.get("LOCALAI_AMD_ATTN_MIX_TILES", "1") == "1"
+
+
+def attn_mix_tiles(q_lens: Sequence[int], device) -> Tuple[torch.Tensor, int]:
+    """Work tiles of attn_mix's matrix-core kernel for the leading sequences of a batch, whose
+    portions hold q_lens rows: ([ntiles, 2] int32 (sequence, first row within its portion), rows
+    covered)."""
+    t = [(s, r) for s, n in enumerate(q_lens) for r in range(0, int(n), ATTN_MIX_QT)]
+    return torch.tensor(t or [(0, 0)], dtype=torch.int32, device=device), int(sum(int(n) for n in q_lens))
+
+
 def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_seq: torch.Tensor, pos: torch.Tensor,
              block_tables: torch.Tensor, H: int, scale: float, softcap: float = 0.0,
              slopes: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None, chunk: int = 0,
-             window: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Attention with reshaped scores over row-major paged K/V ([blocks, G, BS, Dk / Dv]); one
+             window: int = 0, gate: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None,
+             tile_rows: int = 0, cu_q: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention with reshaped scores over paged K ([blocks, G, BS, Dk]) and V ([blocks, G, BS / 8,
+    Dv, 8], transposed per 8 keys: the operand layout of the P.V matrix instruction); one
     query row per token, row r belonging to sequence row_seq[r] (block_tables row) at position
     pos[r], its keys 0..pos[r] already in the pools.  Per head g: s = scale q.k, softcap tanh,
     minus slopes[g] * distance; then the heads' scores are mixed by talk [H, H]; keys are visible
     within the query's chunk of `chunk` positions and the last `window` positions (0: no limit);
     softmax; values of width Dv; each head's output times sigmoid(gate[r, h]) (gate: [T, H] view,
-    any row stride).  Returns [T, H * Dv] in q's dtype; scores and softmax in fp32."""
+    any row stride).  Returns [T, H * Dv] in q's dtype; scores and softmax in fp32.
+    tiles / tile_rows / cu_q (attn_mix_tiles): the first tile_rows rows are whole prompt portions,
+    positions consecutive within each; in bf16 and where the shape allows (key width % 32, value
+    width % 16 and <= 128, at most 32 heads) they run on the matrix-core tile kernel, every other
+    row -- decode rows, fp32, odd shapes -- on the row kernel."""
     T = q.shape[0]
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     Dv = v_cache.shape[3]
+    if v_cache.dim() != 5 or v_cache.shape[2] * 8 != BS or v_cache.shape[4] != 8:
+        raise ValueError("attn_mix: V pages must be [blocks, G, BS / 8, Dv, 8]")
     if q.shape[1] != H * Dk or H % G or row_seq.shape[0] != T or pos.shape[0] != T:
         raise ValueError("attn_mix: operand shapes do not fit")
     if not q.is_cuda:
@@ -1833,7 +1864,7 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
             tab = block_tables[int(row_seq[r])].long()
             blk, off = tab[js // BS], js % BS
             kk = k_cache[blk, :, off].float().repeat_interleave(rep, 1)     # [n, H, Dk]
-            vv = v_cache[blk, :, off].float().repeat_interleave(rep, 1)
+            vv = v_cache[blk, :, off // 8, :, off % 8].float().repeat_interleave(rep, 1)
             s = torch.einsum("hd,nhd->hn", qf[r], kk) * scale
             if softcap > 0:
                 s = softcap * torch.tanh(s / softcap)
@@ -1863,10 +1894,27 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
             raise ValueError("attn_mix: gate must be a [T, H] view of q's dtype with unit column stride")
         ldg = gate.stride(0)
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
-    _check(lib().la_attn_mix_rows(int(f32), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), row_seq.data_ptr(),
-                                  pos.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], T, H, G, Dk, Dv, BS,
-                                  float(scale), float(softcap), _ptr(slopes), _ptr(talk), int(chunk), int(window),
-                                  _ptr(gate), ldg, out.data_ptr(), _stream()), "la_attn_mix_rows")
+    r0 = 0
+    if (tiles is not None and tile_rows > 0 and not f32 and ATTN_MIX_TILES and Dk % 32 == 0 and Dv % 16 == 0
+            and Dv <= 128 and H <= 32):
+        if cu_q is None or tile_rows > T or tiles.dtype != torch.int32 or not tiles.is_contiguous():
+            raise ValueError("attn_mix: tiles need cu_q and int32 [ntiles, 2]")
+        rc = lib().la_attn_mix_tiles(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tiles.data_ptr(),
+                                     tiles.shape[0], cu_q.data_ptr(), pos.data_ptr(), block_tables.data_ptr(),
+                                     block_tables.shape[1], H, G, Dk, Dv, BS, float(scale), float(softcap), _ptr(slopes),
+                                     _ptr(talk), int(chunk), int(window), _ptr(gate), ldg, out.data_ptr(), _stream())
+        if rc == 0:
+            r0 = tile_rows
+        elif rc != 1:
+            _check(rc, "la_attn_mix_tiles")
+    if r0 < T:
+        esz = q.element_size()
+        _check(lib().la_attn_mix_rows(int(f32), q.data_ptr() + r0 * H * Dk * esz, k_cache.data_ptr(),
+                                      v_cache.data_ptr(), row_seq.data_ptr() + r0 * 4, pos.data_ptr() + r0 * 4,
+                                      block_tables.data_ptr(), block_tables.shape[1], T - r0, H, G, Dk, Dv, BS,
+                                      float(scale), float(softcap), _ptr(slopes), _ptr(talk), int(chunk), int(window),
+                                      None if gate is None else gate.data_ptr() + r0 * ldg * esz, ldg,
+                                      out.data_ptr() + r0 * H * Dv * esz, _stream()), "la_attn_mix_rows")
     return out
 
 

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
         float a = acc[e] * alpha[h];
         for (int jj = 0; jj < nk; ++jj) {
           const int j = j0 + jj, blk = tab[j / BS], off = j % BS;
-          a = fmaf(s2[h * AM_KT + jj], (float)vc[(((long)blk * G + g) * BS + off) * Dv + d], a);
+          a = fmaf(s2[h * AM_KT + jj], (float)vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)], a);
         }
         acc[e] = a;
       }
@@ -151,6 +151,215 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
       out[(long)r * HV + o] = (AT)v;
     }
   }
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// Prompt portions in bf16 on the matrix cores.  Workgroup = 16 consecutive query rows of one
+// sequence portion x ALL heads, NW waves; per tile of 32 keys:
+//   A  S_h = Q_h K_g^T per head (heads dealt round-robin to the waves), MFMA 16x16x32 bf16 with
+//      both operands read straight from global memory in operand layout (16 B per lane);
+//      scale, softcap and the distance slope applied to the fp32 accumulators -> LDS s1[h][q][key]
+//   B  head mix s'_h = sum_g talk[h][g] s_g as an fp32 MFMA 16x16x4 (A = talk, B = 16 (q, key)
+//      columns of s1) -- scores never leave fp32 -- written back in place with the visibility mask
+//      (a wave owns its column blocks, and reads all of a block before it writes)
+//   C  one online-softmax step per (head, query) row: a thread per row over the 32 keys;
+//      probabilities -> LDS as bf16 in A-operand layout
+//   D  O_h += P_h V_g, MFMA 16x16x32 bf16, V read from the pages transposed per 8 keys
+// Epilogue: 1 / l, the sigmoid head gate, bf16 store.  HPW = heads per wave, NDV = Dv / 16.
+constexpr int AT_KT = 32;
+constexpr int AT_SS = AT_KT + 1;   // fp32 score row stride: rows spread over the LDS banks
+constexpr int AT_PS = AT_KT + 8;   // bf16 probability row stride: 16-byte aligned rows
+
+template <int NW, int HPW, int NDV>
+__global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ pos,
+    const int* __restrict__ bt, int maxb, int H, int G, int Dk, int Dv, int BS, float scale, float softcap,
+    const float* __restrict__ slopes, const float* __restrict__ talk, int chunk, int window,
+    const bf16* __restrict__ gate, int ldg, bf16* __restrict__ out) {
+  extern __shared__ float lds[];
+  float* s1 = lds;                           // [H][16][AT_SS]
+  float* mrun = s1 + H * 16 * AT_SS;         // [H * 16]
+  float* lrun = mrun + H * 16;
+  float* alpha = lrun + H * 16;
+  bf16* pb = (bf16*)(alpha + H * 16);        // [H][16][AT_PS]
+  const int seq = tiles[2 * blockIdx.x], r0 = tiles[2 * blockIdx.x + 1];
+  const int qbeg = cu_q[seq], qlen = cu_q[seq + 1] - qbeg;
+  const int nrow = min(16, qlen - r0);
+  const int row0 = qbeg + r0;
+  const int pos0 = pos[row0];                // positions of a portion are consecutive
+  const int last = pos0 + nrow - 1;
+  const int* tab = bt + (long)seq * maxb;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fr = lane & 15, fq = lane >> 4;
+  const int rep = H / G, KC = Dk / 32;
+  for (int e = tid; e < H * 16; e += NW * 64) { mrun[e] = -INFINITY; lrun[e] = 0.f; }
+  f32x4 o[HPW][NDV];
+#pragma unroll
+  for (int a = 0; a < HPW; ++a)
+#pragma unroll
+    for (int b = 0; b < NDV; ++b) o[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int lo0 = chunk > 0 ? (pos0 / chunk) * chunk : 0;
+  if (window > 0) lo0 = max(lo0, pos0 - window + 1);
+  __syncthreads();
+  for (int j0 = (lo0 / AT_KT) * AT_KT; j0 <= last; j0 += AT_KT) {
+    // ---- A: raw scores
+#pragma unroll
+    for (int hi = 0; hi < HPW; ++hi) {
+      const int h = wave + NW * hi;
+      if (h >= H) continue;
+      const int g = h / rep;
+      const float slope = slopes ? slopes[h] : 0.f;
+#pragma unroll
+      for (int ns = 0; ns < 2; ++ns) {
+        const int key = j0 + 16 * ns + fr;
+        const bf16* kp = nullptr;
+        if (key <= last) {
+          const int blk = tab[key / BS], off = key % BS;
+          kp = kc + (((long)blk * G + g) * BS + off) * Dk;
+        }
+        const bf16* qp = q + ((long)(row0 + min(fr, nrow - 1)) * H + h) * Dk;
+        f32x4 a = {0.f, 0.f, 0.f, 0.f};
+        for (int kc2 = 0; kc2 < KC; ++kc2) {
+          const bf16x8 qa = *(const bf16x8*)(qp + 32 * kc2 + 8 * fq);
+          bf16x8 kb = {};
+          if (kp) kb = *(const bf16x8*)(kp + 32 * kc2 + 8 * fq);
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb, a, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int qr = 4 * fq + i, qpos = pos0 + qr;
+          float sc = a[i] * scale;
+          if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+          sc -= slope * (float)(qpos - key);
+          if (key > qpos || qr >= nrow) sc = 0.f;   // hidden below; finite for the mix
+          s1[(h * 16 + qr) * AT_SS + 16 * ns + fr] = sc;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- B: head mix (fp32 MFMA) + visibility, in place
+    for (int cb = wave; cb < 2 * 16; cb += NW) {
+      const int qr = cb >> 1, kk = (cb & 1) * 16 + fr;
+      f32x4 acc[4];
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int MB = (H + 15) >> 4;
+      if (talk) {
+        for (int ks = 0; ks < (H + 3) >> 2; ++ks) {
+          const int g = 4 * ks + fq;
+          const float b = g < H ? s1[(g * 16 + qr) * AT_SS + kk] : 0.f;
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb) {
+            if (mb < MB) {
+              const int m = 16 * mb + fr;
+              const float a = (m < H && g < H) ? talk[m * H + g] : 0.f;
+              acc[mb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[mb], 0, 0, 0);
+            }
+          }
+        }
+      }
+      const int key = j0 + kk, qpos = pos0 + qr;
+      int lo = chunk > 0 ? (qpos / chunk) * chunk : 0;
+      if (window > 0) lo = max(lo, qpos - window + 1);
+      const bool vis = qr < nrow && key <= qpos && key >= lo;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        if (mb < MB) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int h = 16 * mb + 4 * fq + i;
+            if (h < H) {
+              float* p = s1 + (h * 16 + qr) * AT_SS + kk;
+              const float v = talk ? acc[mb][i] : *p;
+              *p = vis ? v : -INFINITY;
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // ---- C: online softmax, a thread per (head, query) row
+    for (int r = tid; r < H * 16; r += NW * 64) {
+      const float* sr = s1 + r * AT_SS;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int k = 0; k < AT_KT; ++k) mx = fmaxf(mx, sr[k]);
+      const float mo = mrun[r], mn = fmaxf(mo, mx);
+      float sum = 0.f;
+      bf16* pr = pb + r * AT_PS;
+#pragma unroll
+      for (int k = 0; k < AT_KT; ++k) {
+        const float p = (sr[k] == -INFINITY) ? 0.f : __expf(sr[k] - mn);
+        sum += p;
+        pr[k] = (bf16)p;
+      }
+      const float a = (mo == -INFINITY) ? 0.f : __expf(mo - mn);
+      alpha[r] = a;
+      lrun[r] = lrun[r] * a + sum;
+      mrun[r] = mn;
+    }
+    __syncthreads();
+    // ---- D: O += P V
+#pragma unroll
+    for (int hi = 0; hi < HPW; ++hi) {
+      const int h = wave + NW * hi;
+      if (h >= H) continue;
+      const int g = h / rep;
+      const bf16x8 pa = *(const bf16x8*)(pb + (h * 16 + fr) * AT_PS + 8 * fq);
+      float al[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) al[i] = alpha[h * 16 + 4 * fq + i];
+      const int key8 = j0 + 8 * fq;
+      const bf16* vp = nullptr;
+      if (key8 <= last) {
+        const int blk = tab[key8 / BS], off = key8 % BS;
+        vp = vc + ((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv) * 8;
+      }
+#pragma unroll
+      for (int nd = 0; nd < NDV; ++nd) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[hi][nd][i] *= al[i];
+        const int d = 16 * nd + fr;
+        bf16x8 vb = {};
+        if (vp && d < Dv) vb = *(const bf16x8*)(vp + (long)d * 8);
+        o[hi][nd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[hi][nd], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int hi = 0; hi < HPW; ++hi) {
+    const int h = wave + NW * hi;
+    if (h >= H) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int qr = 4 * fq + i;
+      if (qr >= nrow) continue;
+      const float l = lrun[h * 16 + qr];
+      float f = l > 0.f ? 1.f / l : 0.f;
+      if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)(row0 + qr) * ldg + h]));
+#pragma unroll
+      for (int nd = 0; nd < NDV; ++nd) {
+        const int d = 16 * nd + fr;
+        if (d < Dv) out[((long)(row0 + qr) * H + h) * Dv + d] = (bf16)(o[hi][nd][i] * f);
+      }
+    }
+  }
+}
+
+template <int NW, int HPW, int NDV>
+static int launch_tile(int ntiles, size_t shm, hipStream_t s, const void* q, const void* kc, const void* vc,
+                       const void* tiles, const void* cu_q, const void* pos, const void* bt, int maxb, int H, int G,
+                       int Dk, int Dv, int BS, float scale, float softcap, const void* slopes, const void* talk,
+                       int chunk, int window, const void* gate, int ldg, void* out) {
+  auto k = attn_mix_tile_kernel<NW, HPW, NDV>;
+  if (shm > 48 * 1024) (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+  hipLaunchKernelGGL(k, dim3(ntiles), dim3(NW * 64), shm, s, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,
+                     (const int*)tiles, (const int*)cu_q, (const int*)pos, (const int*)bt, maxb, H, G, Dk, Dv, BS, scale,
+                     softcap, (const float*)slopes, (const float*)talk, chunk, window, (const bf16*)gate, ldg,
+                     (bf16*)out);
+  return (int)hipGetLastError();
 }
 
 }  // namespace la
@@ -180,4 +389,28 @@ extern "C" int la_attn_mix_rows(int f32, const void* q, const void* kc, const vo
                        (bf16*)out);
   }
   return (int)hipGetLastError();
+}
+
+// Prompt portions (bf16): tiles [ntiles][2] = (sequence, first row of the tile within the
+// sequence's portion), 16 rows per tile.  Returns 1 when the shape is outside the kernel's reach
+// (the caller then uses la_attn_mix_rows): Dk % 32, Dv % 16, Dv <= 128, H <= 32, BS % 8.
+extern "C" int la_attn_mix_tiles(const void* q, const void* kc, const void* vc, const void* tiles, int ntiles,
+                                 const void* cu_q, const void* pos, const void* bt, int maxb, int H, int G, int Dk,
+                                 int Dv, int BS, float scale, float softcap, const void* slopes, const void* talk,
+                                 int chunk, int window, const void* gate, int ldg, void* out, void* stream) {
+  using namespace la;
+  if (ntiles <= 0 || H <= 0 || G <= 0 || H % G) return -1;
+  if ((Dk % 32) || (Dv % 16) || Dv > 128 || H > 32 || (BS & 7)) return 1;
+  const size_t shm = (size_t)H * 16 * (AT_SS * 4 + 3 * 4 + AT_PS * 2);
+  if (shm > 150 * 1024) return 1;
+  hipStream_t s = (hipStream_t)stream;
+  const int nw = H > 16 ? 8 : 4, hpw = (H + nw - 1) / nw, ndv = Dv <= 32 ? 2 : (Dv <= 64 ? 4 : 8);
+#define LA_TILE(NW, HPW, NDV)                                                                                      \
+  if (nw == NW && hpw <= HPW && ndv == NDV)                                                                        \
+    return launch_tile<NW, HPW, NDV>(ntiles, shm, s, q, kc, vc, tiles, cu_q, pos, bt, maxb, H, G, Dk, Dv, BS, scale, \
+                                     softcap, slopes, talk, chunk, window, gate, ldg, out);
+  LA_TILE(4, 1, 2) LA_TILE(4, 1, 4) LA_TILE(4, 1, 8) LA_TILE(4, 2, 2) LA_TILE(4, 2, 4) LA_TILE(4, 2, 8)
+  LA_TILE(4, 4, 2) LA_TILE(4, 4, 4) LA_TILE(4, 4, 8) LA_TILE(8, 4, 2) LA_TILE(8, 4, 4) LA_TILE(8, 4, 8)
+#undef LA_TILE
+  return 1;
 }

@@ -10,8 +10,9 @@
 // slot needs no clearing when another sequence takes it over.
 //
 // Outputs: q rows [T, Cq]; k into the paged K pool [blocks, G, BS, Dk]; v -- optionally mixed with
-// the first mixing layer's values, v <- (1 - lam) v + lam v_first -- into the V pool
-// [blocks, G, BS, Dv].  Accumulation, the mix and lam are fp32; storage is the activation type.
+// the first mixing layer's values, v <- (1 - lam) v + lam v_first -- into the V pool, which is
+// transposed per 8 keys, [blocks, G, BS / 8, Dv, 8] (the P.V matrix instruction's operand layout).
+// Accumulation, the mix and lam are fp32; storage is the activation type.
 #include "common.h"
 
 namespace la {
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(256) void shortconv_kv_kernel(
     if (slot >= 0) {
       const int g = cv / Dv, d = cv - g * Dv;
       const int blk = slot / BS, off = slot - blk * BS;
-      vc[(((long)blk * G + g) * BS + off) * Dv + d] = (AT)v;
+      vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)] = (AT)v;
     }
   }
 }
@@ -112,7 +113,7 @@ extern "C" int la_shortconv_kv(int f32, int single, const void* u, int ldp, cons
                                int nseq, void* stream) {
   using namespace la;
   const int C = Cq + Ck + Cv;
-  if (taps < 1 || taps > 9 || T <= 0 || C <= 0 || Ck != G * Dk || Cv != G * Dv || (single && nseq != T)) return -1;
+  if (taps < 1 || taps > 9 || T <= 0 || C <= 0 || Ck != G * Dk || Cv != G * Dv || (single && nseq != T) || (BS & 7)) return -1;
   dim3 grid((C + 255) / 256, T), gs((C + 255) / 256, nseq);
   hipStream_t s = (hipStream_t)stream;
 #define LA_SC(AT, SG)                                                                                          \

@@ -76,7 +76,6 @@ def _time(fn, iters: int) -> float:
 
 
 def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters: int) -> Dict[str, float]:
-    from .. import ops
     from ..engine.llm_engine import EngineConfig, LLMEngine
     from ..models.decoder import DecoderModel, ForwardBatch
     tokens = max(n_seq * prompt, batch * (context + 32))
@@ -103,8 +102,8 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
             fb.seq_lens, fb.max_len = eng._dev(plan["p_ctx"]), int(plan["p_ctx"].max())
         else:
             fb.cu_q, fb.ctx_lens = eng._dev(plan["p_cu"]), eng._dev(plan["p_ctx"])
-            if dm:
-                fb.tiles = ops.prefill_tiles(q.tolist(), eng.device)
+            if not dec:
+                fb.tiles, fb.tile_rows = eng.model.prefill_tiles(q, eng.device)
         if not dm:
             fb.sslots = eng._dev(plan["p_sslot"])
             fb.row_seq = eng._dev(np.repeat(np.arange(k, dtype=np.int32), q))

@@ -37,7 +37,7 @@ def paged(T, BS, rng, extra=3):
 def test_shortconv_portions_state_and_value_mix(device, dtype, taps):
     rng = np.random.default_rng(taps)
     g = torch.Generator().manual_seed(taps)
-    H, G, Dk, Dv, BS = 3, 1, 8, 5, 4
+    H, G, Dk, Dv, BS = 3, 1, 8, 5, 8
     Cq, Ck, Cv = H * Dk, G * Dk, G * Dv
     C = Cq + Ck + Cv
     lens = {0: 11, 1: 6}
@@ -50,7 +50,7 @@ def test_shortconv_portions_state_and_value_mix(device, dtype, taps):
     tab1 = [b for b in range(nblk + 2) if b not in set(tab0.tolist())][:2]
     slots = {0: slots0, 1: [tab1[t // BS] * BS + t % BS for t in range(6)]}
     kc = ops.kv_pages(nblk + 2, G, BS, Dk, dtype, device)
-    vc = ops.kv_pages(nblk + 2, G, BS, Dv, dtype, device)
+    vc = ops.v_pages(nblk + 2, G, BS, Dv, dtype, device)
     # both state slots hold another sequence's leftovers: nothing before position 0 may be read
     state = torch.full((2, taps - 1, C), 1e4, dtype=dtype, device=device)
     wd = w.to(device)
@@ -79,7 +79,7 @@ def test_shortconv_portions_state_and_value_mix(device, dtype, taps):
         assert rel(q_got[s], want[s][:, :Cq]) < tol
         sl = torch.tensor(slots[s])
         k = kc.cpu().float()[sl // BS, :, sl % BS].reshape(len(sl), Ck)
-        v = vc.cpu().float()[sl // BS, :, sl % BS].reshape(len(sl), Cv)
+        v = vc.cpu().float()[sl // BS, :, (sl % BS) // 8, :, sl % 8].reshape(len(sl), Cv)
         assert rel(k, want[s][:, Cq:Cq + Ck]) < tol
         assert rel(v, (1 - 0.37) * want[s][:, Cq + Ck:] + 0.37 * vfirst[s]) < tol
     # the state ends as the last taps - 1 projected rows of each sequence
@@ -107,10 +107,10 @@ def _attn_case(device, dtype, T, H, G, Dk, Dv, BS, chunk, softcap, scale, boost,
     want = oracle.attention(q, k, v, gate, talk, scale, softcap, chunk)
     nblk, table, slots = paged(T, BS, rng)
     kc = ops.kv_pages(nblk, G, BS, Dk, dtype, device)
-    vc = ops.kv_pages(nblk, G, BS, Dv, dtype, device)
+    vc = ops.v_pages(nblk, G, BS, Dv, dtype, device)
     sl = torch.tensor(slots)
     kc[sl // BS, :, sl % BS] = k.to(device=device, dtype=dtype)
-    vc[sl // BS, :, sl % BS] = v.to(device=device, dtype=dtype)
+    vc[sl // BS, :, (sl % BS) // 8, :, sl % 8] = v.to(device=device, dtype=dtype)
     bt = i32([table.tolist(), table.tolist()], device)
     qd = q.reshape(T, H * Dk).to(device=device, dtype=dtype)
     # the gate rides in a wider matrix, as it does beside the projections
@@ -153,9 +153,67 @@ def test_attention_chunk_edges(device, dtype, chunk):
 @pytest.mark.parametrize("device,dtype", MODES)
 def test_attention_shapes_that_the_usual_model_hides(device, dtype):
     # one kv head for six query heads, value wider than key, odd widths (no vector loads), no chunk
-    _attn_case(device, dtype, 41, 6, 1, 5, 11, 4, 0, 4.0, 0.5, [(40, 0, 5)], 13)
+    _attn_case(device, dtype, 41, 6, 1, 5, 11, 8, 0, 4.0, 0.5, [(40, 0, 5)], 13)
     # one head: the head mix is a scalar
     _attn_case(device, dtype, 20, 1, 1, 8, 8, 8, 6, 0.0, 0.3, [], 14)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,Dk,Dv,BS,chunk,softcap", [(4, 2, 64, 32, 16, 40, 20.0), (16, 4, 128, 128, 32, 100, 30.0),
+                                                      (32, 8, 64, 64, 8, 24, 0.0), (3, 1, 32, 16, 16, 0, 10.0),
+                                                      (6, 6, 32, 48, 16, 33, 15.0)])
+def test_attention_tile_kernel_portions(H, G, Dk, Dv, BS, chunk, softcap):
+    """The matrix-core kernel on prompt portions that start mid-sequence (not on a tile, page or
+    chunk border) beside single decode rows in the same launch, two sequences of unequal length,
+    towering keys at the chunk's edges; against the oracle over the whole sequences."""
+    dev, dtype = "cuda:0", torch.bfloat16
+    rng = np.random.default_rng(H)
+    g = torch.Generator().manual_seed(H)
+    lens, starts = [151, 77, 60], [37, 0, 59]          # portion = rows [start, len); the third is one decode row
+    scale = Dk ** -0.5
+    talk = torch.eye(H) + 0.25 * torch.randn(H, H, generator=g)
+    nblk = sum(-(-n // BS) for n in lens) + 2
+    perm = rng.permutation(nblk)
+    kc, vc = ops.kv_pages(nblk, G, BS, Dk, dtype, dev), ops.v_pages(nblk, G, BS, Dv, dtype, dev)
+    maxb = max(-(-n // BS) for n in lens)
+    bt = np.zeros((3, maxb), dtype=np.int32)
+    qs, gates, wants, o = [], [], [], 0
+    for s, (n, a) in enumerate(zip(lens, starts)):
+        q, k, v = torch.randn(n, H, Dk, generator=g), torch.randn(n, G, Dk, generator=g), torch.randn(n, G, Dv, generator=g)
+        c = chunk or n
+        for i in (a, a + 1, n - 1):                      # towering keys: first of the chunk, one before it
+            i = min(i, n - 1)
+            for j, h in (((i // c) * c, 0), ((i // c) * c - 1, H - 1)):
+                if j >= 0:
+                    d = torch.zeros(Dk)
+                    d[(i + j) % Dk] = 5.0
+                    q[i, h] += d / scale ** 0.5
+                    k[j, h // (H // G)] += d / scale ** 0.5
+        q, k, v = (t.to(dtype).float() for t in (q, k, v))
+        gate = torch.randn(n, H, generator=g).to(dtype).float()
+        wants.append(oracle.attention(q, k, v, gate, talk, scale, softcap, chunk)[a:])
+        tab = perm[o:o + -(-n // BS)]
+        o += len(tab)
+        bt[s, :len(tab)] = tab
+        sl = torch.tensor([int(tab[t // BS]) * BS + t % BS for t in range(n)])
+        kc[sl // BS, :, sl % BS] = k.to(device=dev, dtype=dtype)
+        vc[sl // BS, :, (sl % BS) // 8, :, sl % 8] = v.to(device=dev, dtype=dtype)
+        qs.append(q[a:].reshape(n - a, H * Dk))
+        gates.append(gate[a:])
+    rows = [n - a for n, a in zip(lens, starts)]
+    qd = torch.cat(qs).to(device=dev, dtype=dtype)
+    gd = torch.cat(gates).to(device=dev, dtype=dtype)
+    row_seq = i32(np.repeat(np.arange(3), rows), dev)
+    pos = i32(np.concatenate([np.arange(a, n) for n, a in zip(lens, starts)]), dev)
+    cu = i32(np.concatenate([[0], np.cumsum(rows)]), dev)
+    tiles, tile_rows = ops.attn_mix_tiles(rows[:2], dev)
+    assert tile_rows == rows[0] + rows[1]
+    args = dict(H=H, scale=scale, softcap=softcap, slopes=ops.alibi_slopes(H, dev), talk=talk.to(dev), chunk=chunk, gate=gd)
+    got = ops.attn_mix(qd, kc, vc, row_seq, pos, i32(bt, dev), tiles=tiles, tile_rows=tile_rows, cu_q=cu, **args)
+    ref = ops.attn_mix(qd, kc, vc, row_seq, pos, i32(bt, dev), **args)          # the row kernel alone
+    want = torch.cat(wants)
+    assert rel(got, want) < 3e-2 and rel(ref, want) < 3e-2
+    assert rel(got, ref.float().cpu()) < 2e-2
 
 
 @pytest.mark.gpu
