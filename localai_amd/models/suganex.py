@@ -26,6 +26,7 @@ framework's other models) or true fp32 end to end (dtype=torch.float32).
 """
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
@@ -39,6 +40,14 @@ from .decoder import ForwardBatch, KVCache, TPInfo
 # batches of at most this many tokens (and every captured decode graph) run the routed experts as
 # pair GEMVs; larger ones group rows by expert for library GEMMs (one host read of the grouping)
 MOE_PAIR_MAX_T = 32
+# ... and from this many tokens on, where the grouped expert GEMM kernels apply (see _moe)
+MOE_DENSE_MIN_T = 6144
+# decode rows through the matrix-core tile kernel (one-row tiles, split over the keys) instead of the row kernel
+DECODE_TILES = os.environ.get("LOCALAI_AMD_SUGANEX_DECODE_TILES", "1") == "1"
+
+
+def res_is_cuda(fb) -> bool:
+    return fb.tokens.is_cuda
 
 
 @dataclass
@@ -134,6 +143,8 @@ class _Layer:
     wu: Optional[torch.Tensor] = None
     wd: Optional[torch.Tensor] = None          # [E, D, F]
     experts: Optional[list] = None             # [(gate QWeight, up QWeight, down QWeight)]
+    moe_gu: Optional[object] = None            # ops.MoEWeights of the fused gate|up / down projections, where
+    moe_down: Optional[object] = None          # the grouped expert GEMM kernels take the shape (bf16, K % 256 == 0)
 
 
 class SuganexModel:
@@ -178,6 +189,8 @@ class SuganexModel:
             raise ValueError("suganex: embed shape does not fit config vocab / width")
         self.layers: List[_Layer] = []
         self.v_first_layer = next((i for i, m in enumerate(hp.mixers) if m.v_mix), -1)
+        if len({m.Cv for m in hp.mixers if m.v_mix}) > 1:
+            raise ValueError("suganex: layers that mix values must share kv_heads * vdim")
         for i, (m, f) in enumerate(zip(hp.mixers, hp.mlps)):
             p = f"l{i}."
             H = m.heads
@@ -213,6 +226,12 @@ class SuganexModel:
                     raise ValueError(f"layer {i}: expert shapes do not fit the config")
                 L.wg, L.wu, L.wd = (t.to(device=device, dtype=dtype).contiguous() for t in (g, u, d))
                 L.experts = [(qw(L.wg[e]), qw(L.wu[e]), qw(L.wd[e])) for e in range(f.experts)]
+                if not self.f32 and device.type == "cuda" and D % 256 == 0 and f.ff % 256 == 0:
+                    # the framework's grouped expert GEMMs (one weight stream per active expert, device
+                    # routing, no host sync) read [gate; up] fused per expert
+                    gu = torch.cat([L.wg, L.wu], 1).contiguous()
+                    L.moe_gu = ops.MoEWeights([ops.QWeight.from_float(gu[e]) for e in range(f.experts)])
+                    L.moe_down = ops.MoEWeights([d_ for _, _, d_ in L.experts])
             self.layers.append(L)
         self.out_norm = 1.0 + f32("final.norm")
         self.output = qw(raw("head"))
@@ -237,10 +256,12 @@ class SuganexModel:
         return ops.attn_mix_tiles(q_lens, device)
 
     def _single_rows(self, T: int):
+        """(row -> sequence, row ranges, one-row work tiles) of a batch with one row per sequence."""
         a = self._aranges.get(T)
         if a is None:
             r = torch.arange(T + 1, dtype=torch.int32, device=self.device)
-            a = self._aranges[T] = (r[:T].contiguous(), r)
+            tiles = torch.stack([r[:T], torch.zeros_like(r[:T])], 1).contiguous()
+            a = self._aranges[T] = (r[:T].contiguous(), r, tiles)
         return a
 
     # --------------------------------------------------------------------------- forward
@@ -270,6 +291,13 @@ class SuganexModel:
         T = xn.shape[0]
         ids, wts = ops.router_sigmoid(xn, L.router, L.corr, f.top, True)
         capturing = xn.is_cuda and torch.cuda.is_current_stream_capturing()
+        if L.moe_gu is not None and (T < MOE_DENSE_MIN_T or capturing) and T > 2:
+            # grouped expert GEMMs on the routed rows, as the Mixtral path: gate|up, SiLU gating, then
+            # the down projection whose routing-weighted slabs the next add_norm sums
+            order, off = ops.moe_route(ids, f.experts)
+            gu = ops.moe_linear(xn, L.moe_gu, order, off, f.top, T)
+            h = ops.act(gu, f.ff, ops.ACT_SWIGLU)
+            return ops.moe_linear(h, L.moe_down, order, off, f.top, T, down=True, wts=wts)
         if T <= MOE_PAIR_MAX_T or capturing:
             return ops.Partial(ops.moe_pairs(xn, L.wg, L.wu, L.wd, ids, wts).unsqueeze(0))
         # rows grouped by expert (device), one host read of the group offsets, then per expert
@@ -309,13 +337,16 @@ class SuganexModel:
         if kv.state is None or fb.sslots is None:
             raise ValueError("suganex: the batch needs state slots (engine built without a state pool?)")
         if fb.decode:
-            row_seq, cu_q = self._single_rows(T)
+            row_seq, cu_q, tiles = self._single_rows(T)
+            tile_rows = T if (DECODE_TILES and not self.f32 and res_is_cuda(fb)) else 0
             single = True
+            splits_for = lambda m: max(1, min(16, 512 // max(T, 1), -(-(m.chunk or fb.max_len or 1) // 32)))  # noqa: E731
         else:
-            row_seq, cu_q = fb.row_seq, fb.cu_q
+            row_seq, cu_q, tiles, tile_rows = fb.row_seq, fb.cu_q, fb.tiles, fb.tile_rows
             if row_seq is None:
                 raise ValueError("suganex: prompt batches need fb.row_seq")
             single = False
+            splits_for = lambda m: 1  # noqa: E731
         res = ops.embed(fb.tokens, self.tok_embd)
         if not res.is_contiguous() or res.dtype != torch.float32:
             res = res.float().contiguous()
@@ -334,7 +365,7 @@ class SuganexModel:
                                  kv.state[i], kv.k[i], kv.v[i], vfirst_in=vin, vfirst_out=vout, lam=lam, single=single)
             a = ops.attn_mix(q, kv.k[i], kv.v[i], row_seq, fb.pos, fb.block_tables, m.heads, m.scale, m.softcap,
                              L.slopes, L.talk, m.chunk, m.window, gate=proj[:, C:C + m.heads],
-                             tiles=None if fb.decode else fb.tiles, tile_rows=fb.tile_rows, cu_q=cu_q)
+                             tiles=tiles, tile_rows=tile_rows, cu_q=cu_q, key_splits=splits_for(m))
             o = ops.linear(a, L.wo)
             nxt = self.layers[i + 1].norm1 if i + 1 < n else self.out_norm
             if f is not None:

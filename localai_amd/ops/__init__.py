@@ -121,7 +121,7 @@ def lib():
             "la_decode_advance": [P, P, P, P, P, P, I, I, I, P, I, P, P, P],
             "la_shortconv_kv": [I, I, P, I, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, P, P, P, I, I, P],
             "la_attn_mix_rows": [I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
-            "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
+            "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, I, P, P, I, P],
             "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
             "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
@@ -1831,7 +1831,7 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
              block_tables: torch.Tensor, H: int, scale: float, softcap: float = 0.0,
              slopes: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None, chunk: int = 0,
              window: int = 0, gate: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None,
-             tile_rows: int = 0, cu_q: Optional[torch.Tensor] = None) -> torch.Tensor:
+             tile_rows: int = 0, cu_q: Optional[torch.Tensor] = None, key_splits: int = 1) -> torch.Tensor:
     """Attention with reshaped scores over paged K ([blocks, G, BS, Dk]) and V ([blocks, G, BS / 8,
     Dv, 8], transposed per 8 keys: the operand layout of the P.V matrix instruction); one
     query row per token, row r belonging to sequence row_seq[r] (block_tables row) at position
@@ -1843,7 +1843,9 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     tiles / tile_rows / cu_q (attn_mix_tiles): the first tile_rows rows are whole prompt portions,
     positions consecutive within each; in bf16 and where the shape allows (key width % 32, value
     width % 16 and <= 128, at most 32 heads) they run on the matrix-core tile kernel, every other
-    row -- decode rows, fp32, odd shapes -- on the row kernel."""
+    row -- fp32, odd shapes, rows after tile_rows -- on the row kernel.  key_splits > 1 deals every
+    tile's keys to that many workgroups and merges their partial results in a second launch: for
+    batches of few rows with many keys each (decoding)."""
     T = q.shape[0]
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     Dv = v_cache.shape[3]
@@ -1899,10 +1901,16 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
             and Dv <= 128 and H <= 32):
         if cu_q is None or tile_rows > T or tiles.dtype != torch.int32 or not tiles.is_contiguous():
             raise ValueError("attn_mix: tiles need cu_q and int32 [ntiles, 2]")
+        ns = max(1, min(int(key_splits), 64))
+        po = pml = None
+        if ns > 1:
+            po = torch.empty(tile_rows * H * ns * Dv, dtype=torch.float32, device=q.device)
+            pml = torch.empty(tile_rows * H * ns * 2, dtype=torch.float32, device=q.device)
         rc = lib().la_attn_mix_tiles(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tiles.data_ptr(),
                                      tiles.shape[0], cu_q.data_ptr(), pos.data_ptr(), block_tables.data_ptr(),
                                      block_tables.shape[1], H, G, Dk, Dv, BS, float(scale), float(softcap), _ptr(slopes),
-                                     _ptr(talk), int(chunk), int(window), _ptr(gate), ldg, out.data_ptr(), _stream())
+                                     _ptr(talk), int(chunk), int(window), _ptr(gate), ldg, out.data_ptr(), ns,
+                                     _ptr(po), _ptr(pml), tile_rows, _stream())
         if rc == 0:
             r0 = tile_rows
         elif rc != 1:

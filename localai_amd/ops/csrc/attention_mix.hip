@@ -157,8 +157,9 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
 // ------------------------------------------------------------------------------------------------
 // Prompt portions in bf16 on the matrix cores.  Workgroup = 16 consecutive query rows of one
 // sequence portion x ALL heads, NW waves; per tile of 32 keys:
-//   A  S_h = Q_h K_g^T per head (heads dealt round-robin to the waves), MFMA 16x16x32 bf16 with
-//      both operands read straight from global memory in operand layout (16 B per lane);
+//   A  S_h = Q_h K_g^T per head (a wave owns HPW consecutive heads, so heads of one kv group
+//      share their K fragments), MFMA 16x16x32 bf16 with both operands read straight from global
+//      memory in operand layout (16 B per lane), Q fragments kept in registers over the key loop;
 //      scale, softcap and the distance slope applied to the fp32 accumulators -> LDS s1[h][q][key]
 //   B  head mix s'_h = sum_g talk[h][g] s_g as an fp32 MFMA 16x16x4 (A = talk, B = 16 (q, key)
 //      columns of s1) -- scores never leave fp32 -- written back in place with the visibility mask
@@ -177,7 +178,8 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ pos,
     const int* __restrict__ bt, int maxb, int H, int G, int Dk, int Dv, int BS, float scale, float softcap,
     const float* __restrict__ slopes, const float* __restrict__ talk, int chunk, int window,
-    const bf16* __restrict__ gate, int ldg, bf16* __restrict__ out) {
+    const bf16* __restrict__ gate, int ldg, bf16* __restrict__ out, int nsplit, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
   extern __shared__ float lds[];
   float* s1 = lds;                           // [H][16][AT_SS]
   float* mrun = s1 + H * 16 * AT_SS;         // [H * 16]
@@ -199,42 +201,91 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   for (int a = 0; a < HPW; ++a)
 #pragma unroll
     for (int b = 0; b < NDV; ++b) o[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // a wave owns HPW consecutive heads: heads of one kv group share their K and V fragments.
+  // Q fragments (A operand: row fr, k = 32 kc + 8 fq) stay in registers for the whole key loop
+  // where the register file allows (one wave per SIMD); keys wider than 128 are re-read.
+  constexpr bool QREG = NW == 4 && HPW * NDV <= 16;
+  const int h0 = wave * HPW;
+  bf16x8 qa[QREG ? HPW : 1][4];
+  if constexpr (QREG) {
+#pragma unroll
+    for (int hi = 0; hi < HPW; ++hi)
+#pragma unroll
+      for (int kc2 = 0; kc2 < 4; ++kc2) {
+        bf16x8 v = {};
+        if (h0 + hi < H && kc2 < KC)
+          v = *(const bf16x8*)(q + ((long)(row0 + min(fr, nrow - 1)) * H + h0 + hi) * Dk + 32 * kc2 + 8 * fq);
+        qa[hi][kc2] = v;
+      }
+  }
   int lo0 = chunk > 0 ? (pos0 / chunk) * chunk : 0;
   if (window > 0) lo0 = max(lo0, pos0 - window + 1);
   __syncthreads();
-  for (int j0 = (lo0 / AT_KT) * AT_KT; j0 <= last; j0 += AT_KT) {
+  // blockIdx.y = key split: every nsplit-th key tile (decode rows: few query rows, many keys)
+  for (int j0 = (lo0 / AT_KT + (int)blockIdx.y) * AT_KT; j0 <= last; j0 += AT_KT * nsplit) {
     // ---- A: raw scores
+    for (int kb0 = 0; kb0 < KC; kb0 += 4) {      // key widths beyond 128: 128 at a time
+      bf16x8 kf[2][4];
+      int gprev = -1;
+      // one head: (re)load its group's K fragments, 8 MFMAs per 16 keys x 128 columns, scores -> LDS
+      auto head = [&](int hi, int h, auto&& qfrag) {
+        const int g = h / rep;
+        if (g != gprev) {                          // this group's K fragments (B operand: key fr, k = 32 kc + 8 fq)
+          gprev = g;
 #pragma unroll
-    for (int hi = 0; hi < HPW; ++hi) {
-      const int h = wave + NW * hi;
-      if (h >= H) continue;
-      const int g = h / rep;
-      const float slope = slopes ? slopes[h] : 0.f;
+          for (int ns = 0; ns < 2; ++ns) {
+            const int key = j0 + 16 * ns + fr;
+            const bf16* kp = nullptr;
+            if (key <= last) {
+              const int blk = tab[key / BS], off = key % BS;
+              kp = kc + (((long)blk * G + g) * BS + off) * Dk;
+            }
 #pragma unroll
-      for (int ns = 0; ns < 2; ++ns) {
-        const int key = j0 + 16 * ns + fr;
-        const bf16* kp = nullptr;
-        if (key <= last) {
-          const int blk = tab[key / BS], off = key % BS;
-          kp = kc + (((long)blk * G + g) * BS + off) * Dk;
+            for (int kc2 = 0; kc2 < 4; ++kc2) {
+              bf16x8 v = {};
+              if (kp && kb0 + kc2 < KC) v = *(const bf16x8*)(kp + 32 * (kb0 + kc2) + 8 * fq);
+              kf[ns][kc2] = v;
+            }
+          }
         }
+        const float slope = slopes ? slopes[h] : 0.f;
         const bf16* qp = q + ((long)(row0 + min(fr, nrow - 1)) * H + h) * Dk;
-        f32x4 a = {0.f, 0.f, 0.f, 0.f};
-        for (int kc2 = 0; kc2 < KC; ++kc2) {
-          const bf16x8 qa = *(const bf16x8*)(qp + 32 * kc2 + 8 * fq);
-          bf16x8 kb = {};
-          if (kp) kb = *(const bf16x8*)(kp + 32 * kc2 + 8 * fq);
-          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb, a, 0, 0, 0);
-        }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int qr = 4 * fq + i, qpos = pos0 + qr;
-          float sc = a[i] * scale;
-          if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-          sc -= slope * (float)(qpos - key);
-          if (key > qpos || qr >= nrow) sc = 0.f;   // hidden below; finite for the mix
-          s1[(h * 16 + qr) * AT_SS + 16 * ns + fr] = sc;
+        for (int ns = 0; ns < 2; ++ns) {
+          f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kc2 = 0; kc2 < 4; ++kc2) {
+            if (kb0 + kc2 < KC)
+              a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag(qp, kc2), kf[ns][kc2], a, 0, 0, 0);
+          }
+          const int key = j0 + 16 * ns + fr;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int qr = 4 * fq + i;
+            float* sp = s1 + (h * 16 + qr) * AT_SS + 16 * ns + fr;
+            if (kb0 > 0) a[i] += *sp;              // partial dot products of the earlier 128 columns
+            if (kb0 + 4 < KC) { *sp = a[i]; continue; }
+            const int qpos = pos0 + qr;
+            float sc = a[i] * scale;
+            if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+            sc -= slope * (float)(qpos - key);
+            if (key > qpos || qr >= nrow) sc = 0.f;   // hidden below; finite for the mix
+            *sp = sc;
+          }
         }
+      };
+      if constexpr (QREG) {
+#pragma unroll
+        for (int hi = 0; hi < HPW; ++hi)
+          if (h0 + hi < H)
+            head(hi, h0 + hi, [&](const bf16* qp, int kc2) {
+              return kb0 == 0 ? qa[hi][kc2] : *(const bf16x8*)(qp + 32 * (kb0 + kc2) + 8 * fq);
+            });
+      } else {
+#pragma unroll 1
+        for (int hi = 0; hi < HPW; ++hi)
+          if (h0 + hi < H)
+            head(hi, h0 + hi, [&](const bf16* qp, int kc2) { return *(const bf16x8*)(qp + 32 * (kb0 + kc2) + 8 * fq); });
       }
     }
     __syncthreads();
@@ -300,42 +351,70 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
       mrun[r] = mn;
     }
     __syncthreads();
-    // ---- D: O += P V
-#pragma unroll
-    for (int hi = 0; hi < HPW; ++hi) {
-      const int h = wave + NW * hi;
-      if (h >= H) continue;
-      const int g = h / rep;
-      const bf16x8 pa = *(const bf16x8*)(pb + (h * 16 + fr) * AT_PS + 8 * fq);
-      float al[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) al[i] = alpha[h * 16 + 4 * fq + i];
+    // ---- D: O += P V; a V fragment (B operand: channel fr, keys 8 fq ..) serves every head of its group
+    {
+      bf16x8 pa[HPW];
       const int key8 = j0 + 8 * fq;
-      const bf16* vp = nullptr;
-      if (key8 <= last) {
-        const int blk = tab[key8 / BS], off = key8 % BS;
-        vp = vc + ((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv) * 8;
+      int blk8 = -1, off8 = 0;
+      if (key8 <= last) { blk8 = tab[key8 / BS]; off8 = key8 % BS; }
+#pragma unroll
+      for (int hi = 0; hi < HPW; ++hi) {
+        const int h = h0 + hi;
+        bf16x8 v = {};
+        if (h < H) {
+          v = *(const bf16x8*)(pb + (h * 16 + fr) * AT_PS + 8 * fq);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float al = alpha[h * 16 + 4 * fq + i];
+#pragma unroll
+            for (int nd = 0; nd < NDV; ++nd) o[hi][nd][i] *= al;
+          }
+        }
+        pa[hi] = v;
       }
 #pragma unroll
       for (int nd = 0; nd < NDV; ++nd) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[hi][nd][i] *= al[i];
         const int d = 16 * nd + fr;
         bf16x8 vb = {};
-        if (vp && d < Dv) vb = *(const bf16x8*)(vp + (long)d * 8);
-        o[hi][nd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[hi][nd], 0, 0, 0);
+        int gprev = -1;
+#pragma unroll
+        for (int hi = 0; hi < HPW; ++hi) {
+          const int h = h0 + hi;
+          if (h >= H) continue;
+          const int g = h / rep;
+          if (g != gprev) {
+            gprev = g;
+            vb = bf16x8{};
+            if (blk8 >= 0 && d < Dv)
+              vb = *(const bf16x8*)(vc + (((((long)blk8 * G + g) * (BS >> 3) + (off8 >> 3)) * Dv) + d) * 8);
+          }
+          o[hi][nd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[hi], vb, o[hi][nd], 0, 0, 0);
+        }
       }
     }
   }
   __syncthreads();
 #pragma unroll
   for (int hi = 0; hi < HPW; ++hi) {
-    const int h = wave + NW * hi;
+    const int h = h0 + hi;
     if (h >= H) continue;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int qr = 4 * fq + i;
       if (qr >= nrow) continue;
+      if (nsplit > 1) {   // unnormalised partial result of this key split; attn_mix_merge_kernel finishes
+        const long base = ((long)(row0 + qr) * H + h) * nsplit + blockIdx.y;
+        if (fr == 0) {
+          part_ml[2 * base] = mrun[h * 16 + qr];
+          part_ml[2 * base + 1] = lrun[h * 16 + qr];
+        }
+#pragma unroll
+        for (int nd = 0; nd < NDV; ++nd) {
+          const int d = 16 * nd + fr;
+          if (d < Dv) part_o[base * Dv + d] = o[hi][nd][i];
+        }
+        continue;
+      }
       const float l = lrun[h * 16 + qr];
       float f = l > 0.f ? 1.f / l : 0.f;
       if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)(row0 + qr) * ldg + h]));
@@ -348,17 +427,42 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   }
 }
 
+// out[row][h][d] = gate * sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the key splits
+__global__ __launch_bounds__(256) void attn_mix_merge_kernel(const float* __restrict__ part_o,
+                                                             const float* __restrict__ part_ml, int nsplit, int H, int Dv,
+                                                             const bf16* __restrict__ gate, int ldg,
+                                                             bf16* __restrict__ out) {
+  const int row = blockIdx.x;
+  for (int e = threadIdx.x; e < H * Dv; e += 256) {
+    const int h = e / Dv, d = e - h * Dv;
+    const long base = ((long)row * H + h) * nsplit;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
+    float L = 0.f, acc = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float m = part_ml[2 * (base + s)];
+      if (m == -INFINITY) continue;
+      const float w = __expf(m - M);
+      L = fmaf(part_ml[2 * (base + s) + 1], w, L);
+      acc = fmaf(part_o[(base + s) * Dv + d], w, acc);
+    }
+    float f = L > 0.f ? 1.f / L : 0.f;
+    if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)row * ldg + h]));
+    out[((long)row * H + h) * Dv + d] = (bf16)(acc * f);
+  }
+}
+
 template <int NW, int HPW, int NDV>
-static int launch_tile(int ntiles, size_t shm, hipStream_t s, const void* q, const void* kc, const void* vc,
+static int launch_tile(int nsplit, void* part_o, void* part_ml, int ntiles, size_t shm, hipStream_t s, const void* q, const void* kc, const void* vc,
                        const void* tiles, const void* cu_q, const void* pos, const void* bt, int maxb, int H, int G,
                        int Dk, int Dv, int BS, float scale, float softcap, const void* slopes, const void* talk,
                        int chunk, int window, const void* gate, int ldg, void* out) {
   auto k = attn_mix_tile_kernel<NW, HPW, NDV>;
   if (shm > 48 * 1024) (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
-  hipLaunchKernelGGL(k, dim3(ntiles), dim3(NW * 64), shm, s, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,
+  hipLaunchKernelGGL(k, dim3(ntiles, nsplit), dim3(NW * 64), shm, s, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,
                      (const int*)tiles, (const int*)cu_q, (const int*)pos, (const int*)bt, maxb, H, G, Dk, Dv, BS, scale,
                      softcap, (const float*)slopes, (const float*)talk, chunk, window, (const bf16*)gate, ldg,
-                     (bf16*)out);
+                     (bf16*)out, nsplit, (float*)part_o, (float*)part_ml);
   return (int)hipGetLastError();
 }
 
@@ -394,23 +498,34 @@ extern "C" int la_attn_mix_rows(int f32, const void* q, const void* kc, const vo
 // Prompt portions (bf16): tiles [ntiles][2] = (sequence, first row of the tile within the
 // sequence's portion), 16 rows per tile.  Returns 1 when the shape is outside the kernel's reach
 // (the caller then uses la_attn_mix_rows): Dk % 32, Dv % 16, Dv <= 128, H <= 32, BS % 8.
+// nsplit > 1 (batches of few rows with many keys, i.e. decoding): every tile's keys are dealt to
+// nsplit workgroups whose partial results (part_o [rows, H, nsplit, Dv], part_ml [rows, H, nsplit, 2],
+// fp32, rows = the batch rows the tiles cover) a second launch merges.
 extern "C" int la_attn_mix_tiles(const void* q, const void* kc, const void* vc, const void* tiles, int ntiles,
                                  const void* cu_q, const void* pos, const void* bt, int maxb, int H, int G, int Dk,
                                  int Dv, int BS, float scale, float softcap, const void* slopes, const void* talk,
-                                 int chunk, int window, const void* gate, int ldg, void* out, void* stream) {
+                                 int chunk, int window, const void* gate, int ldg, void* out, int nsplit, void* part_o,
+                                 void* part_ml, int rows, void* stream) {
   using namespace la;
-  if (ntiles <= 0 || H <= 0 || G <= 0 || H % G) return -1;
+  if (ntiles <= 0 || H <= 0 || G <= 0 || H % G || nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml)))
+    return -1;
   if ((Dk % 32) || (Dv % 16) || Dv > 128 || H > 32 || (BS & 7)) return 1;
   const size_t shm = (size_t)H * 16 * (AT_SS * 4 + 3 * 4 + AT_PS * 2);
   if (shm > 150 * 1024) return 1;
   hipStream_t s = (hipStream_t)stream;
   const int nw = H > 16 ? 8 : 4, hpw = (H + nw - 1) / nw, ndv = Dv <= 32 ? 2 : (Dv <= 64 ? 4 : 8);
+  int rc = 1;
 #define LA_TILE(NW, HPW, NDV)                                                                                      \
-  if (nw == NW && hpw <= HPW && ndv == NDV)                                                                        \
-    return launch_tile<NW, HPW, NDV>(ntiles, shm, s, q, kc, vc, tiles, cu_q, pos, bt, maxb, H, G, Dk, Dv, BS, scale, \
-                                     softcap, slopes, talk, chunk, window, gate, ldg, out);
+  if (rc == 1 && nw == NW && hpw <= HPW && ndv == NDV)                                                             \
+    rc = launch_tile<NW, HPW, NDV>(nsplit, part_o, part_ml, ntiles, shm, s, q, kc, vc, tiles, cu_q, pos, bt, maxb, H, \
+                                   G, Dk, Dv, BS, scale, softcap, slopes, talk, chunk, window, gate, ldg, out);
   LA_TILE(4, 1, 2) LA_TILE(4, 1, 4) LA_TILE(4, 1, 8) LA_TILE(4, 2, 2) LA_TILE(4, 2, 4) LA_TILE(4, 2, 8)
   LA_TILE(4, 4, 2) LA_TILE(4, 4, 4) LA_TILE(4, 4, 8) LA_TILE(8, 4, 2) LA_TILE(8, 4, 4) LA_TILE(8, 4, 8)
 #undef LA_TILE
-  return 1;
+  if (rc == 0 && nsplit > 1) {
+    hipLaunchKernelGGL(attn_mix_merge_kernel, dim3(rows), dim3(256), 0, s, (const float*)part_o, (const float*)part_ml,
+                       nsplit, H, Dv, (const bf16*)gate, ldg, (bf16*)out);
+    rc = (int)hipGetLastError();
+  }
+  return rc;
 }

@@ -6,7 +6,8 @@ checkpoint) and routed experts (Suganex vs a Mixtral-style checkpoint), both sto
 weights so every GEMM takes the same library path -- and each is timed through its engine's own
 batch construction (native scheduler, paged KV pool, state slots) and `model.forward`:
   prefill: `n_seq` prompts of `prompt` tokens in one batch, tokens/s;
-  decode:  `batch` sequences holding `context` tokens each, one token per sequence and step, tokens/s.
+  decode:  `batch` sequences holding `context` tokens each, one token per sequence and step, tokens/s
+           (1536 by default: a Suganex row then sees the 513 keys of its chunk of 1024, a llama row all 1537).
 The forward is repeated on the same batch (it rewrites the same K/V slots), so the numbers are the
 kernels' and the GEMMs', without the host's planning time.
 """
@@ -96,9 +97,9 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
         k, q = len(ids), plan["p_qlen"]
         dec = bool(plan["p_decode"].all()) and n == 1
         fb = ForwardBatch(tokens=eng._dev(plan["p_tokens"]), pos=eng._dev(plan["p_pos"]), slots=eng._dev(plan["p_slots"]),
-                          decode=dec and dm, block_tables=eng._dev(plan["p_bt"]),
+                          decode=dec, block_tables=eng._dev(plan["p_bt"]),
                           logits_idx=eng._dev(np.asarray(plan["p_cu"][1:] - 1, dtype=np.int64)))
-        if dec and dm:
+        if dec:
             fb.seq_lens, fb.max_len = eng._dev(plan["p_ctx"]), int(plan["p_ctx"].max())
         else:
             fb.cu_q, fb.ctx_lens = eng._dev(plan["p_cu"]), eng._dev(plan["p_ctx"])
@@ -133,7 +134,7 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
 
 
 def run(design: str, sizes: List[str], cache: str, n_seq: int = 4, prompt: int = 2048, batch: int = 64,
-        context: int = 1024, iters: int = 5) -> dict:
+        context: int = 1536, iters: int = 5) -> dict:
     if design != "suganex":
         raise SystemExit(f"--design-compare: unknown design {design!r} (suganex)")
     os.makedirs(cache, exist_ok=True)

@@ -53,6 +53,12 @@ CONFIGS = {
         layer(mixer(heads=3, kv=3, dim=16, vdim=8, conv=3, chunk=33, scale=0.25, softcap=5.0, v_mix=False), dense(40)),
         layer(mixer(heads=6, kv=1, dim=8, vdim=16, conv=4, chunk=7, scale=0.3, softcap=30.0), moe(32, 6, 3)),
         layer(mixer(heads=6, kv=1, dim=8, vdim=16, conv=2, chunk=64, scale=0.2, softcap=12.0), dense(72))]},
+    # widths the GPU's specialised paths take: key width % 32 and value width % 16 (matrix-core
+    # attention tiles), GEMM depths % 256 (skinny / grouped expert GEMMs)
+    "wide": {"vocab": 97, "width": 256, "norm": {"eps": 1e-6}, "layers": [
+        layer(mixer(heads=4, kv=2, dim=32, vdim=16, conv=4, chunk=20, scale=0.18, softcap=25.0), moe(256, 4, 2)),
+        layer(mixer(heads=8, kv=2, dim=64, vdim=32, conv=3, chunk=48, scale=0.125, softcap=0.0, v_mix=False), dense(512)),
+        layer(mixer(heads=4, kv=2, dim=32, vdim=16, conv=2, chunk=20, scale=0.18, softcap=25.0), None)]},
 }
 
 
@@ -166,7 +172,7 @@ def rand_tokens(cfg, n, seed):
 
 # --------------------------------------------------------------------------------------- whole prompts
 @pytest.mark.parametrize("device,dtype", MODES)
-@pytest.mark.parametrize("name", ["small", "varied"])
+@pytest.mark.parametrize("name", ["small", "varied", "wide"])
 def test_whole_prompt_matches_oracle(ckpt, name, device, dtype):
     path, cfg, W = ckpt(name)
     toks = rand_tokens(cfg, 70, 1)            # several chunks of every layer, pages of 16
@@ -203,8 +209,9 @@ def test_residual_stream_after_every_layer(ckpt, device):
 
 # --------------------------------------------------------------------------------------- portions, decoding
 @pytest.mark.parametrize("device,dtype", MODES)
-def test_portions_and_token_by_token_decoding(ckpt, device, dtype):
-    path, cfg, W = ckpt("varied")
+@pytest.mark.parametrize("name", ["varied", "wide"])
+def test_portions_and_token_by_token_decoding(ckpt, name, device, dtype):
+    path, cfg, W = ckpt(name)
     toks = rand_tokens(cfg, 90, 3)
     want = oracle.forward(cfg, W, toks)
     eng = engine(path, device, dtype)
@@ -224,11 +231,12 @@ def test_long_decoding_over_chunks_and_pages(ckpt, device, dtype):
 
 # --------------------------------------------------------------------------------------- batches, reuse
 @pytest.mark.parametrize("device,dtype", MODES)
-def test_mixed_batches_of_unequal_requests_with_page_and_slot_reuse(ckpt, device, dtype):
+@pytest.mark.parametrize("name", ["varied", "wide"])
+def test_mixed_batches_of_unequal_requests_with_page_and_slot_reuse(ckpt, name, device, dtype):
     """Four live requests at most in a pool of 160 tokens with 4 state slots, ten requests in all:
     portions of some beside single tokens of others, every finished request's pages and slot taken
     over by the next.  Every position must equal the request run alone (the oracle)."""
-    path, cfg, W = ckpt("varied")
+    path, cfg, W = ckpt(name)
     rng = np.random.default_rng(5)
     lens = [33, 7, 48, 2, 21, 40, 1, 17, 30, 9]
     reqs = {i + 1: rand_tokens(cfg, n, 100 + i) for i, n in enumerate(lens)}

@@ -214,6 +214,13 @@ def test_attention_tile_kernel_portions(H, G, Dk, Dv, BS, chunk, softcap):
     want = torch.cat(wants)
     assert rel(got, want) < 3e-2 and rel(ref, want) < 3e-2
     assert rel(got, ref.float().cpu()) < 2e-2
+    # every tile's keys dealt to several workgroups and merged (how decode batches run), the lone
+    # decode row included as a one-row tile
+    tiles_all, n_all = ops.attn_mix_tiles(rows, dev)
+    for splits in (2, 5):
+        got2 = ops.attn_mix(qd, kc, vc, row_seq, pos, i32(bt, dev), tiles=tiles_all, tile_rows=n_all, cu_q=cu,
+                            key_splits=splits, **args)
+        assert rel(got2, want) < 3e-2 and rel(got2, ref.float().cpu()) < 2e-2
 
 
 @pytest.mark.gpu
