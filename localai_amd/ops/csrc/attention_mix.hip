@@ -204,7 +204,7 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   // a wave owns HPW consecutive heads: heads of one kv group share their K and V fragments.
   // Q fragments (A operand: row fr, k = 32 kc + 8 fq) stay in registers for the whole key loop
   // where the register file allows (one wave per SIMD); keys wider than 128 are re-read.
-  constexpr bool QREG = NW == 4 && HPW * NDV <= 16;
+  constexpr bool QREG = HPW * NDV <= 8;
   const int h0 = wave * HPW;
   bf16x8 qa[QREG ? HPW : 1][4];
   if constexpr (QREG) {
@@ -225,16 +225,17 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   for (int j0 = (lo0 / AT_KT + (int)blockIdx.y) * AT_KT; j0 <= last; j0 += AT_KT * nsplit) {
     // ---- A: raw scores
     for (int kb0 = 0; kb0 < KC; kb0 += 4) {      // key widths beyond 128: 128 at a time
-      bf16x8 kf[2][4];
-      int gprev = -1;
-      // one head: (re)load its group's K fragments, 8 MFMAs per 16 keys x 128 columns, scores -> LDS
-      auto head = [&](int hi, int h, auto&& qfrag) {
-        const int g = h / rep;
-        if (g != gprev) {                          // this group's K fragments (B operand: key fr, k = 32 kc + 8 fq)
-          gprev = g;
-#pragma unroll
-          for (int ns = 0; ns < 2; ++ns) {
-            const int key = j0 + 16 * ns + fr;
+      // 16 keys at a time: this wave's heads against their group's K fragments (B operand: key fr,
+      // k = 32 kc + 8 fq), reloaded only when the kv group changes from one head to the next
+#pragma unroll 1
+      for (int ns = 0; ns < 2; ++ns) {
+        bf16x8 kf[4];
+        int gprev = -1;
+        const int key = j0 + 16 * ns + fr;
+        auto head = [&](int h, auto&& qfrag) {
+          const int g = h / rep;
+          if (g != gprev) {
+            gprev = g;
             const bf16* kp = nullptr;
             if (key <= last) {
               const int blk = tab[key / BS], off = key % BS;
@@ -244,21 +245,16 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
             for (int kc2 = 0; kc2 < 4; ++kc2) {
               bf16x8 v = {};
               if (kp && kb0 + kc2 < KC) v = *(const bf16x8*)(kp + 32 * (kb0 + kc2) + 8 * fq);
-              kf[ns][kc2] = v;
+              kf[kc2] = v;
             }
           }
-        }
-        const float slope = slopes ? slopes[h] : 0.f;
-        const bf16* qp = q + ((long)(row0 + min(fr, nrow - 1)) * H + h) * Dk;
-#pragma unroll
-        for (int ns = 0; ns < 2; ++ns) {
+          const float slope = slopes ? slopes[h] : 0.f;
+          const bf16* qp = q + ((long)(row0 + min(fr, nrow - 1)) * H + h) * Dk;
           f32x4 a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int kc2 = 0; kc2 < 4; ++kc2) {
-            if (kb0 + kc2 < KC)
-              a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag(qp, kc2), kf[ns][kc2], a, 0, 0, 0);
+            if (kb0 + kc2 < KC) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag(qp, kc2), kf[kc2], a, 0, 0, 0);
           }
-          const int key = j0 + 16 * ns + fr;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int qr = 4 * fq + i;
@@ -272,20 +268,20 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
             if (key > qpos || qr >= nrow) sc = 0.f;   // hidden below; finite for the mix
             *sp = sc;
           }
-        }
-      };
-      if constexpr (QREG) {
+        };
+        if constexpr (QREG) {
 #pragma unroll
-        for (int hi = 0; hi < HPW; ++hi)
-          if (h0 + hi < H)
-            head(hi, h0 + hi, [&](const bf16* qp, int kc2) {
-              return kb0 == 0 ? qa[hi][kc2] : *(const bf16x8*)(qp + 32 * (kb0 + kc2) + 8 * fq);
-            });
-      } else {
+          for (int hi = 0; hi < HPW; ++hi)
+            if (h0 + hi < H)
+              head(h0 + hi, [&](const bf16* qp, int kc2) {
+                return kb0 == 0 ? qa[hi][kc2] : *(const bf16x8*)(qp + 32 * (kb0 + kc2) + 8 * fq);
+              });
+        } else {
 #pragma unroll 1
-        for (int hi = 0; hi < HPW; ++hi)
-          if (h0 + hi < H)
-            head(hi, h0 + hi, [&](const bf16* qp, int kc2) { return *(const bf16x8*)(qp + 32 * (kb0 + kc2) + 8 * fq); });
+          for (int hi = 0; hi < HPW; ++hi)
+            if (h0 + hi < H)
+              head(h0 + hi, [&](const bf16* qp, int kc2) { return *(const bf16x8*)(qp + 32 * (kb0 + kc2) + 8 * fq); });
+        }
       }
     }
     __syncthreads();
@@ -334,12 +330,12 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
     for (int r = tid; r < H * 16; r += NW * 64) {
       const float* sr = s1 + r * AT_SS;
       float mx = -INFINITY;
-#pragma unroll
+#pragma unroll 8
       for (int k = 0; k < AT_KT; ++k) mx = fmaxf(mx, sr[k]);
       const float mo = mrun[r], mn = fmaxf(mo, mx);
       float sum = 0.f;
       bf16* pr = pb + r * AT_PS;
-#pragma unroll
+#pragma unroll 8
       for (int k = 0; k < AT_KT; ++k) {
         const float p = (sr[k] == -INFINITY) ? 0.f : __expf(sr[k] - mn);
         sum += p;
@@ -428,26 +424,27 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
 }
 
 // out[row][h][d] = gate * sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the key splits
-__global__ __launch_bounds__(256) void attn_mix_merge_kernel(const float* __restrict__ part_o,
+__global__ __launch_bounds__(128) void attn_mix_merge_kernel(const float* __restrict__ part_o,
                                                              const float* __restrict__ part_ml, int nsplit, int H, int Dv,
                                                              const bf16* __restrict__ gate, int ldg,
                                                              bf16* __restrict__ out) {
-  const int row = blockIdx.x;
-  for (int e = threadIdx.x; e < H * Dv; e += 256) {
-    const int h = e / Dv, d = e - h * Dv;
-    const long base = ((long)row * H + h) * nsplit;
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
-    float L = 0.f, acc = 0.f;
+  const int row = blockIdx.x, h = blockIdx.y;
+  const long base = ((long)row * H + h) * nsplit;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
+  float L = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float m = part_ml[2 * (base + s)];
+    if (m != -INFINITY) L = fmaf(part_ml[2 * (base + s) + 1], __expf(m - M), L);
+  }
+  float f = L > 0.f ? 1.f / L : 0.f;
+  if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)row * ldg + h]));
+  for (int d = threadIdx.x; d < Dv; d += 128) {
+    float acc = 0.f;
     for (int s = 0; s < nsplit; ++s) {
       const float m = part_ml[2 * (base + s)];
-      if (m == -INFINITY) continue;
-      const float w = __expf(m - M);
-      L = fmaf(part_ml[2 * (base + s) + 1], w, L);
-      acc = fmaf(part_o[(base + s) * Dv + d], w, acc);
+      if (m != -INFINITY) acc = fmaf(part_o[(base + s) * Dv + d], __expf(m - M), acc);
     }
-    float f = L > 0.f ? 1.f / L : 0.f;
-    if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)row * ldg + h]));
     out[((long)row * H + h) * Dv + d] = (bf16)(acc * f);
   }
 }
@@ -513,17 +510,18 @@ extern "C" int la_attn_mix_tiles(const void* q, const void* kc, const void* vc, 
   const size_t shm = (size_t)H * 16 * (AT_SS * 4 + 3 * 4 + AT_PS * 2);
   if (shm > 150 * 1024) return 1;
   hipStream_t s = (hipStream_t)stream;
-  const int nw = H > 16 ? 8 : 4, hpw = (H + nw - 1) / nw, ndv = Dv <= 32 ? 2 : (Dv <= 64 ? 4 : 8);
+  // 8 waves from 9 heads on: fewer heads (accumulator registers) per wave, more waves to hide latency
+  const int nw = H > 8 ? 8 : 4, hpw = (H + nw - 1) / nw, ndv = Dv <= 32 ? 2 : (Dv <= 64 ? 4 : 8);
   int rc = 1;
 #define LA_TILE(NW, HPW, NDV)                                                                                      \
   if (rc == 1 && nw == NW && hpw <= HPW && ndv == NDV)                                                             \
     rc = launch_tile<NW, HPW, NDV>(nsplit, part_o, part_ml, ntiles, shm, s, q, kc, vc, tiles, cu_q, pos, bt, maxb, H, \
                                    G, Dk, Dv, BS, scale, softcap, slopes, talk, chunk, window, gate, ldg, out);
   LA_TILE(4, 1, 2) LA_TILE(4, 1, 4) LA_TILE(4, 1, 8) LA_TILE(4, 2, 2) LA_TILE(4, 2, 4) LA_TILE(4, 2, 8)
-  LA_TILE(4, 4, 2) LA_TILE(4, 4, 4) LA_TILE(4, 4, 8) LA_TILE(8, 4, 2) LA_TILE(8, 4, 4) LA_TILE(8, 4, 8)
+  LA_TILE(8, 2, 2) LA_TILE(8, 2, 4) LA_TILE(8, 2, 8) LA_TILE(8, 4, 2) LA_TILE(8, 4, 4) LA_TILE(8, 4, 8)
 #undef LA_TILE
   if (rc == 0 && nsplit > 1) {
-    hipLaunchKernelGGL(attn_mix_merge_kernel, dim3(rows), dim3(256), 0, s, (const float*)part_o, (const float*)part_ml,
+    hipLaunchKernelGGL(attn_mix_merge_kernel, dim3(rows, H), dim3(128), 0, s, (const float*)part_o, (const float*)part_ml,
                        nsplit, H, Dv, (const bf16*)gate, ldg, (bf16*)out);
     rc = (int)hipGetLastError();
   }

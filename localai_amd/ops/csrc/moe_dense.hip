@@ -20,11 +20,35 @@ __global__ __launch_bounds__(256) void router_sigmoid_kernel(const AT* __restric
   const int t = blockIdx.x * 4 + w;
   const bool live = t < T;
   const AT* xr = x + (long)(live ? t : 0) * ldx;
-  for (int e = 0; e < E; ++e) {
-    float a = 0.f;
-    for (int d = lane; d < D; d += 64) a = fmaf(router[(long)e * D + d], (float)xr[d], a);
-    a = wave_sum(a);
-    if (lane == 0) sc[w][e] = 1.f / (1.f + __expf(-a));
+  // 8 experts at a time: x is read once per pass and the 8 router rows give independent loads
+  for (int e0 = 0; e0 < E; e0 += 8) {
+    float a[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] = 0.f;
+    if ((D & 3) == 0) {
+      for (int d = lane * 4; d < D; d += 256) {
+        const float x0 = (float)xr[d], x1 = (float)xr[d + 1], x2 = (float)xr[d + 2], x3 = (float)xr[d + 3];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if (e0 + k < E) {
+            const float4 r = *(const float4*)(router + (long)(e0 + k) * D + d);
+            a[k] = fmaf(r.x, x0, fmaf(r.y, x1, fmaf(r.z, x2, fmaf(r.w, x3, a[k]))));
+          }
+        }
+      }
+    } else {
+      for (int d = lane; d < D; d += 64) {
+        const float xv = (float)xr[d];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (e0 + k < E) a[k] = fmaf(router[(long)(e0 + k) * D + d], xv, a[k]);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float v = wave_sum(a[k]);
+      if (lane == 0 && e0 + k < E) sc[w][e0 + k] = 1.f / (1.f + __expf(-v));
+    }
   }
   __syncthreads();
   float sum = 0.f, my_s = 0.f;

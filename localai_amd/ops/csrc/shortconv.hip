@@ -82,6 +82,77 @@ __global__ __launch_bounds__(256) void shortconv_kv_kernel(
   }
 }
 
+// bf16 with every width a multiple of 8: one thread per 8 consecutive channels, 16-byte loads of
+// the projection rows and the state, 16-byte stores of q, k and the state (v stays element-wise:
+// its pages are transposed per 8 keys).  Same arithmetic as shortconv_kv_kernel.
+template <bool SINGLE>
+__global__ __launch_bounds__(256) void shortconv_kv8_kernel(
+    const bf16* __restrict__ u, int ldp, const float* __restrict__ w, int taps, int Cq, int Ck, int Cv,
+    const int* __restrict__ row_seq, const int* __restrict__ cu_q, const int* __restrict__ pos,
+    const int* __restrict__ slots, const int* __restrict__ sslot, bf16* __restrict__ state,
+    bf16* __restrict__ q_out, bf16* __restrict__ kc, bf16* __restrict__ vc, int G, int Dk, int Dv, int BS,
+    const float* __restrict__ vfirst_in, float* __restrict__ vfirst_out, const float* __restrict__ lam_p) {
+  const int r = blockIdx.y;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const int C = Cq + Ck + Cv;
+  if (c >= C) return;
+  const int seq = row_seq[r];
+  const int m = r - cu_q[seq];
+  const int p = pos[r];
+  const int ss = sslot[seq];
+  bf16* st = state + (long)ss * (taps - 1) * C + c;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int d = taps - 1 - j;
+    bf16x8 x = {};
+    if (d <= p) {
+      if (d <= m) x = *(const bf16x8*)(u + (long)(r - d) * ldp + c);
+      else if (ss >= 0) x = *(const bf16x8*)(st + (long)(taps - 1 - (d - m)) * C);
+    }
+    if (SINGLE && ss >= 0 && j >= 1) *(bf16x8*)(st + (long)(j - 1) * C) = x;   // row j - 1 <- old row j (or u for the last)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[(long)(c + e) * taps + j], (float)x[e], acc[e]);
+  }
+  const int slot = slots[r];
+  if (c < Cq) {
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)acc[e];
+    *(bf16x8*)(q_out + (long)r * Cq + c) = o;
+  } else if (c < Cq + Ck) {
+    if (slot >= 0) {
+      const int ck = c - Cq, g = ck / Dk, d = ck - g * Dk;
+      const int blk = slot / BS, off = slot - blk * BS;
+      bf16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (bf16)acc[e];
+      *(bf16x8*)(kc + (((long)blk * G + g) * BS + off) * Dk + d) = o;
+    }
+  } else {
+    const int cv = c - Cq - Ck;
+    if (vfirst_out) {
+      *(float4*)(vfirst_out + (long)r * Cv + cv) = float4{acc[0], acc[1], acc[2], acc[3]};
+      *(float4*)(vfirst_out + (long)r * Cv + cv + 4) = float4{acc[4], acc[5], acc[6], acc[7]};
+    }
+    if (vfirst_in) {
+      const float lam = *lam_p;
+      const float4 a = *(const float4*)(vfirst_in + (long)r * Cv + cv), b = *(const float4*)(vfirst_in + (long)r * Cv + cv + 4);
+      const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = (1.f - lam) * acc[e] + lam * f[e];
+    }
+    if (slot >= 0) {
+      const int g = cv / Dv, d = cv - g * Dv;
+      const int blk = slot / BS, off = slot - blk * BS;
+      bf16* vp = vc + ((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vp[e * 8] = (bf16)acc[e];
+    }
+  }
+}
+
 // New tail of every sequence of the batch: the last taps - 1 projected rows up to the end of its
 // portion.  Rows the portion does not cover shift down from the old tail (ascending order: each
 // read is of a higher index than any write before it).
@@ -121,7 +192,19 @@ extern "C" int la_shortconv_kv(int f32, int single, const void* u, int ldp, cons
                      taps, Cq, Ck, Cv, (const int*)row_seq, (const int*)cu_q, (const int*)pos,                \
                      (const int*)slots, (const int*)sslot, (AT*)state, (AT*)q_out, (AT*)kc, (AT*)vc, G, Dk,   \
                      Dv, BS, (const float*)vfirst_in, (float*)vfirst_out, (const float*)lam)
-  if (f32) {
+  const bool vec8 = !f32 && !(Cq & 7) && !(Dk & 7) && !(Dv & 7) && !(ldp & 7) && !((uintptr_t)u & 15) &&
+                    !((uintptr_t)state & 15) && !((uintptr_t)kc & 15) && !((uintptr_t)vfirst_in & 15) &&
+                    !((uintptr_t)vfirst_out & 15);
+  if (vec8) {
+    dim3 g8((C / 8 + 255) / 256, T);
+#define LA_SC8(SG)                                                                                              \
+  hipLaunchKernelGGL((shortconv_kv8_kernel<SG>), g8, dim3(256), 0, s, (const bf16*)u, ldp, (const float*)w, taps, \
+                     Cq, Ck, Cv, (const int*)row_seq, (const int*)cu_q, (const int*)pos, (const int*)slots,      \
+                     (const int*)sslot, (bf16*)state, (bf16*)q_out, (bf16*)kc, (bf16*)vc, G, Dk, Dv, BS,         \
+                     (const float*)vfirst_in, (float*)vfirst_out, (const float*)lam)
+    if (single) LA_SC8(true); else LA_SC8(false);
+#undef LA_SC8
+  } else if (f32) {
     if (single) LA_SC(float, true); else LA_SC(float, false);
   } else {
     if (single) LA_SC(bf16, true); else LA_SC(bf16, false);
