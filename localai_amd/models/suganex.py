@@ -200,7 +200,7 @@ class SuganexModel:
             if (tuple(wq.shape), tuple(wk.shape), tuple(wv.shape), tuple(wg.shape)) != (
                     (m.Cq, D), (m.Ck, D), (m.Cv, D), (H, D)):
                 raise ValueError(f"layer {i}: projection shapes do not fit the config")
-            if m.taps > 1:
+            if m.taps > 1 or p + "mix.q.conv" in T:      # one tap is a per-channel scale
                 conv = torch.cat([raw(p + "mix.q.conv"), raw(p + "mix.k.conv"), raw(p + "mix.v.conv")], 0)
             else:
                 conv = torch.ones(m.Cq + m.Ck + m.Cv, 1)
@@ -271,9 +271,16 @@ class SuganexModel:
             return p.t if p.t.dtype == self.dtype else p.t.to(self.dtype)
         if p.t.dim() == 3 and p.t.shape[0] == 1 and p.bias is None:
             return p.t[0] if self.f32 else p.t[0].to(self.dtype)
+        if p.t.is_cuda and p.N % 4:       # the slab-sum kernel moves 4 columns per thread
+            return p.dense().to(self.dtype)
         return ops.reduce(p, dtype=self.dtype)
 
     def _norm(self, res: torch.Tensor, add, w: torch.Tensor) -> torch.Tensor:
+        if res.is_cuda and res.shape[1] % 4:   # widths the fused kernel does not take: the same steps unfused
+            if add is not None:
+                res += add.dense()
+            y = res * torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + self.hp.norm_eps) * w
+            return y if self.f32 else y.to(torch.bfloat16)
         if not self.f32:
             return ops.add_norm(res, add, w, None, self.hp.norm_eps, 0)
         y = torch.empty_like(res)
@@ -347,7 +354,10 @@ class SuganexModel:
                 raise ValueError("suganex: prompt batches need fb.row_seq")
             single = False
             splits_for = lambda m: 1  # noqa: E731
-        res = ops.embed(fb.tokens, self.tok_embd)
+        if fb.tokens.is_cuda and hp.n_embd % 8:   # the embedding kernel reads 8 columns per thread
+            res = self.tok_embd.materialize_bf16().index_select(0, fb.tokens.long()).float()
+        else:
+            res = ops.embed(fb.tokens, self.tok_embd)
         if not res.is_contiguous() or res.dtype != torch.float32:
             res = res.float().contiguous()
         vfirst = None

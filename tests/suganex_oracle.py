@@ -102,7 +102,7 @@ def forward(cfg, W, tokens, layers_out=None):
         H, G, Dk, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
         h = rms_norm(x, W[p + "norm1"], eps)
         q, k, v = h @ W[p + "mix.q"].T, h @ W[p + "mix.k"].T, h @ W[p + "mix.v"].T
-        if m.get("conv", 1) > 1:
+        if p + "mix.q.conv" in W:
             q, k, v = (short_conv(q, W[p + "mix.q.conv"]), short_conv(k, W[p + "mix.k.conv"]),
                        short_conv(v, W[p + "mix.v.conv"]))
         if m.get("v_mix"):

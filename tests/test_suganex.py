@@ -53,6 +53,11 @@ CONFIGS = {
         layer(mixer(heads=3, kv=3, dim=16, vdim=8, conv=3, chunk=33, scale=0.25, softcap=5.0, v_mix=False), dense(40)),
         layer(mixer(heads=6, kv=1, dim=8, vdim=16, conv=4, chunk=7, scale=0.3, softcap=30.0), moe(32, 6, 3)),
         layer(mixer(heads=6, kv=1, dim=8, vdim=16, conv=2, chunk=64, scale=0.2, softcap=12.0), dense(72))]},
+    # sizes no vector load or fused kernel likes (width % 8 != 0, ff % 4 != 0), a one-tap convolution
+    # (a per-channel scale), five taps, every expert chosen, no mask
+    "odd": {"vocab": 51, "width": 36, "norm": {"eps": 1e-6}, "layers": [
+        layer(mixer(heads=3, kv=1, dim=12, vdim=10, conv=5, chunk=11, scale=0.3, softcap=0.0), dense(30)),
+        layer(mixer(heads=3, kv=3, dim=12, vdim=10, conv=1, chunk=0, scale=0.3, softcap=9.0, v_mix=False), moe(10, 3, 3))]},
     # widths the GPU's specialised paths take: key width % 32 and value width % 16 (matrix-core
     # attention tiles), GEMM depths % 256 (skinny / grouped expert GEMMs)
     "wide": {"vocab": 97, "width": 256, "norm": {"eps": 1e-6}, "layers": [
@@ -172,7 +177,7 @@ def rand_tokens(cfg, n, seed):
 
 # --------------------------------------------------------------------------------------- whole prompts
 @pytest.mark.parametrize("device,dtype", MODES)
-@pytest.mark.parametrize("name", ["small", "varied", "wide"])
+@pytest.mark.parametrize("name", ["small", "varied", "wide", "odd"])
 def test_whole_prompt_matches_oracle(ckpt, name, device, dtype):
     path, cfg, W = ckpt(name)
     toks = rand_tokens(cfg, 70, 1)            # several chunks of every layer, pages of 16
@@ -209,7 +214,7 @@ def test_residual_stream_after_every_layer(ckpt, device):
 
 # --------------------------------------------------------------------------------------- portions, decoding
 @pytest.mark.parametrize("device,dtype", MODES)
-@pytest.mark.parametrize("name", ["varied", "wide"])
+@pytest.mark.parametrize("name", ["varied", "wide", "odd"])
 def test_portions_and_token_by_token_decoding(ckpt, name, device, dtype):
     path, cfg, W = ckpt(name)
     toks = rand_tokens(cfg, 90, 3)
