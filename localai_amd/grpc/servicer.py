@@ -171,7 +171,9 @@ class EngineServicer:
                 mmproj=self._mmproj_path(request, path),
                 lora_adapters=self._lora(request, path),
                 draft_model=self._draft_path(request, path),
-                quantization=str(request.Quantization or "") if is_hf_checkpoint(path) else "")
+                quantization=str(request.Quantization or "") if is_hf_checkpoint(path) else "",
+                # serving precision of families with a 32-bit mode (EngineConfig.dtype)
+                dtype=os.environ.get("LOCALAI_AMD_DTYPE", "bfloat16"))
             loop = asyncio.get_running_loop()
             eng = await loop.run_in_executor(None, lambda: LLMEngine(cfg, tp=self.tp))
             await loop.run_in_executor(None, eng.warmup)
