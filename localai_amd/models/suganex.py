@@ -46,6 +46,10 @@ MOE_DENSE_MIN_T = 6144
 DECODE_TILES = os.environ.get("LOCALAI_AMD_SUGANEX_DECODE_TILES", "1") == "1"
 
 
+# ... with the keys of a row dealt to about this many workgroups per batch
+DECODE_WGS = int(os.environ.get("LOCALAI_AMD_SUGANEX_DECODE_WGS", "512"))
+
+
 def res_is_cuda(fb) -> bool:
     return fb.tokens.is_cuda
 
@@ -130,6 +134,7 @@ class _Layer:
     norm1: torch.Tensor
     qkvg: ops.QWeight                 # [Cq + Ck + Cv + H, D]: q | k | v | gate rows
     conv: torch.Tensor                # [Cq + Ck + Cv, taps] fp32
+    conv_t: torch.Tensor              # the same tap-major, [taps, Cq + Ck + Cv]
     lam: Optional[torch.Tensor]       # [1] fp32 (v_mix layers after the first)
     talk: torch.Tensor                # [H, H] fp32
     slopes: torch.Tensor              # [H] fp32
@@ -210,7 +215,7 @@ class SuganexModel:
             if m.v_mix and i != self.v_first_layer:
                 lam = raw(p + "mix.vmix").reshape(1).to(device).contiguous()
             L = _Layer(norm1=(1.0 + f32(p + "norm1")), qkvg=qw(torch.cat([wq, wk, wv, wg], 0)),
-                       conv=conv.to(device).contiguous(), lam=lam, talk=f32(p + "mix.talk"),
+                       conv=conv.to(device).contiguous(), conv_t=conv.t().contiguous().to(device), lam=lam, talk=f32(p + "mix.talk"),
                        slopes=ops.alibi_slopes(H, device), wo=qw(raw(p + "mix.o")))
             if f is not None:
                 L.norm2 = 1.0 + f32(p + "norm2")
@@ -347,7 +352,7 @@ class SuganexModel:
             row_seq, cu_q, tiles = self._single_rows(T)
             tile_rows = T if (DECODE_TILES and not self.f32 and res_is_cuda(fb)) else 0
             single = True
-            splits_for = lambda m: max(1, min(16, 512 // max(T, 1), -(-(m.chunk or fb.max_len or 1) // 32)))  # noqa: E731
+            splits_for = lambda m: max(1, min(32, DECODE_WGS // max(T, 1), -(-(m.chunk or fb.max_len or 1) // 32)))  # noqa: E731
         else:
             row_seq, cu_q, tiles, tile_rows = fb.row_seq, fb.cu_q, fb.tiles, fb.tile_rows
             if row_seq is None:
@@ -372,7 +377,8 @@ class SuganexModel:
             elif m.v_mix:
                 vin, lam = vfirst, L.lam
             q = ops.shortconv_kv(proj, L.conv, m.Cq, m.Ck, m.Cv, row_seq, cu_q, fb.pos, fb.slots, fb.sslots,
-                                 kv.state[i], kv.k[i], kv.v[i], vfirst_in=vin, vfirst_out=vout, lam=lam, single=single)
+                                 kv.state[i], kv.k[i], kv.v[i], vfirst_in=vin, vfirst_out=vout, lam=lam, single=single,
+                                 w_t=L.conv_t)
             a = ops.attn_mix(q, kv.k[i], kv.v[i], row_seq, fb.pos, fb.block_tables, m.heads, m.scale, m.softcap,
                              L.slopes, L.talk, m.chunk, m.window, gate=proj[:, C:C + m.heads],
                              tiles=tiles, tile_rows=tile_rows, cu_q=cu_q, key_splits=splits_for(m))

@@ -119,7 +119,7 @@ def lib():
             "la_bsgemm_glu": [I, P, P, P, I, P, P, P, I, I, I, P, I, I, P, I, I, I, P],
             "la_bsmoe": [I, I, P, I, I, I, P, P, I, P, I, I, I, P, P, I, LNG, I, I, P],
             "la_decode_advance": [P, P, P, P, P, P, I, I, I, P, I, P, P, P],
-            "la_shortconv_kv": [I, I, P, I, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, P, P, P, I, I, P],
+            "la_shortconv_kv": [I, I, P, I, P, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, P, P, P, I, I, P],
             "la_attn_mix_rows": [I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
             "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, I, P, P, I, P],
             "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
@@ -1734,8 +1734,10 @@ def shortconv_kv(u: torch.Tensor, w: torch.Tensor, Cq: int, Ck: int, Cv: int, ro
                  cu_q: torch.Tensor, pos: torch.Tensor, slots: torch.Tensor, sslot: torch.Tensor,
                  state: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  vfirst_in: Optional[torch.Tensor] = None, vfirst_out: Optional[torch.Tensor] = None,
-                 lam: Optional[torch.Tensor] = None, single: bool = False) -> torch.Tensor:
-    """Depthwise causal convolution over time (w [C, taps] fp32, C = Cq + Ck + Cv) on the first C
+                 lam: Optional[torch.Tensor] = None, single: bool = False,
+                 w_t: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Depthwise causal convolution over time (w [C, taps] fp32, C = Cq + Ck + Cv; w_t: the same
+    weights tap-major, [taps, C], which the vectorised bf16 kernel reads -- made per call when not given) on the first C
     columns of the projection rows u [T, >= C]; rows of one sequence portion are consecutive
     (row_seq [T] -> sequence, cu_q [nseq + 1] row ranges, pos [T] positions).  What precedes a
     portion comes from state[sslot[seq]] ([slots, taps - 1, C]: the last taps - 1 projected rows),
@@ -1802,7 +1804,11 @@ def shortconv_kv(u: torch.Tensor, w: torch.Tensor, Cq: int, Ck: int, Cv: int, ro
         assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (T, Cv))
     assert (vfirst_in is None) == (lam is None) and (lam is None or lam.dtype == torch.float32)
     q = torch.empty(T, Cq, dtype=u.dtype, device=u.device)
-    _check(lib().la_shortconv_kv(int(f32), int(single), u.data_ptr(), u.stride(0), w.data_ptr(), taps, Cq, Ck, Cv,
+    if w_t is None and not f32:
+        w_t = w.t().contiguous()
+    if w_t is not None and (w_t.dtype != torch.float32 or tuple(w_t.shape) != (taps, C) or not w_t.is_contiguous()):
+        raise ValueError("shortconv_kv: w_t must be the fp32 [taps, C] transpose of w")
+    _check(lib().la_shortconv_kv(int(f32), int(single), u.data_ptr(), u.stride(0), w.data_ptr(), _ptr(w_t), taps, Cq, Ck, Cv,
                                  row_seq.data_ptr(), cu_q.data_ptr(), pos.data_ptr(), slots.data_ptr(),
                                  sslot.data_ptr(), state.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                                  v_cache.data_ptr(), G, Dk, Dv, BS, _ptr(vfirst_in), _ptr(vfirst_out), _ptr(lam), T,

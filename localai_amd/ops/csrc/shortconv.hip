@@ -84,10 +84,11 @@ __global__ __launch_bounds__(256) void shortconv_kv_kernel(
 
 // bf16 with every width a multiple of 8: one thread per 8 consecutive channels, 16-byte loads of
 // the projection rows and the state, 16-byte stores of q, k and the state (v stays element-wise:
-// its pages are transposed per 8 keys).  Same arithmetic as shortconv_kv_kernel.
+// its pages are transposed per 8 keys).  Same arithmetic as shortconv_kv_kernel; the weights come
+// tap-major, wt [taps, C], so a thread's 8 weights of one tap are two 16-byte loads.
 template <bool SINGLE>
 __global__ __launch_bounds__(256) void shortconv_kv8_kernel(
-    const bf16* __restrict__ u, int ldp, const float* __restrict__ w, int taps, int Cq, int Ck, int Cv,
+    const bf16* __restrict__ u, int ldp, const float* __restrict__ wt, int taps, int Cq, int Ck, int Cv,
     const int* __restrict__ row_seq, const int* __restrict__ cu_q, const int* __restrict__ pos,
     const int* __restrict__ slots, const int* __restrict__ sslot, bf16* __restrict__ state,
     bf16* __restrict__ q_out, bf16* __restrict__ kc, bf16* __restrict__ vc, int G, int Dk, int Dv, int BS,
@@ -112,8 +113,11 @@ __global__ __launch_bounds__(256) void shortconv_kv8_kernel(
       else if (ss >= 0) x = *(const bf16x8*)(st + (long)(taps - 1 - (d - m)) * C);
     }
     if (SINGLE && ss >= 0 && j >= 1) *(bf16x8*)(st + (long)(j - 1) * C) = x;   // row j - 1 <- old row j (or u for the last)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[(long)(c + e) * taps + j], (float)x[e], acc[e]);
+    const float4 w0 = *(const float4*)(wt + (long)j * C + c), w1 = *(const float4*)(wt + (long)j * C + c + 4);
+    acc[0] = fmaf(w0.x, (float)x[0], acc[0]); acc[1] = fmaf(w0.y, (float)x[1], acc[1]);
+    acc[2] = fmaf(w0.z, (float)x[2], acc[2]); acc[3] = fmaf(w0.w, (float)x[3], acc[3]);
+    acc[4] = fmaf(w1.x, (float)x[4], acc[4]); acc[5] = fmaf(w1.y, (float)x[5], acc[5]);
+    acc[6] = fmaf(w1.z, (float)x[6], acc[6]); acc[7] = fmaf(w1.w, (float)x[7], acc[7]);
   }
   const int slot = slots[r];
   if (c < Cq) {
@@ -177,7 +181,8 @@ __global__ __launch_bounds__(256) void shortconv_state_kernel(const AT* __restri
 
 // f32: 1 = fp32 activations / cache / state, 0 = bf16.  single: every sequence brings exactly one
 // row (decode batches): the state update is fused into the convolution launch.
-extern "C" int la_shortconv_kv(int f32, int single, const void* u, int ldp, const void* w, int taps, int Cq, int Ck,
+// wt: the weights once more, tap-major [taps, C] (may be null: then the scalar kernel runs)
+extern "C" int la_shortconv_kv(int f32, int single, const void* u, int ldp, const void* w, const void* wt, int taps, int Cq, int Ck,
                                int Cv, const void* row_seq, const void* cu_q, const void* pos, const void* slots,
                                const void* sslot, void* state, void* q_out, void* kc, void* vc, int G, int Dk,
                                int Dv, int BS, const void* vfirst_in, void* vfirst_out, const void* lam, int T,
@@ -192,13 +197,13 @@ extern "C" int la_shortconv_kv(int f32, int single, const void* u, int ldp, cons
                      taps, Cq, Ck, Cv, (const int*)row_seq, (const int*)cu_q, (const int*)pos,                \
                      (const int*)slots, (const int*)sslot, (AT*)state, (AT*)q_out, (AT*)kc, (AT*)vc, G, Dk,   \
                      Dv, BS, (const float*)vfirst_in, (float*)vfirst_out, (const float*)lam)
-  const bool vec8 = !f32 && !(Cq & 7) && !(Dk & 7) && !(Dv & 7) && !(ldp & 7) && !((uintptr_t)u & 15) &&
+  const bool vec8 = !f32 && wt && !((uintptr_t)wt & 15) && !(Cq & 7) && !(Dk & 7) && !(Dv & 7) && !(ldp & 7) && !((uintptr_t)u & 15) &&
                     !((uintptr_t)state & 15) && !((uintptr_t)kc & 15) && !((uintptr_t)vfirst_in & 15) &&
                     !((uintptr_t)vfirst_out & 15);
   if (vec8) {
     dim3 g8((C / 8 + 255) / 256, T);
 #define LA_SC8(SG)                                                                                              \
-  hipLaunchKernelGGL((shortconv_kv8_kernel<SG>), g8, dim3(256), 0, s, (const bf16*)u, ldp, (const float*)w, taps, \
+  hipLaunchKernelGGL((shortconv_kv8_kernel<SG>), g8, dim3(256), 0, s, (const bf16*)u, ldp, (const float*)wt, taps, \
                      Cq, Ck, Cv, (const int*)row_seq, (const int*)cu_q, (const int*)pos, (const int*)slots,      \
                      (const int*)sslot, (bf16*)state, (bf16*)q_out, (bf16*)kc, (bf16*)vc, G, Dk, Dv, BS,         \
                      (const float*)vfirst_in, (float*)vfirst_out, (const float*)lam)
