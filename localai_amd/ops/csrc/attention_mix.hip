@@ -204,7 +204,7 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   // a wave owns HPW consecutive heads: heads of one kv group share their K and V fragments.
   // Q fragments (A operand: row fr, k = 32 kc + 8 fq) stay in registers for the whole key loop
   // where the register file allows (one wave per SIMD); keys wider than 128 are re-read.
-  constexpr bool QREG = HPW * NDV <= 8;
+  constexpr bool QREG = HPW * NDV <= 8 || (NW == 8 && HPW == 2);
   const int h0 = wave * HPW;
   bf16x8 qa[QREG ? HPW : 1][4];
   if constexpr (QREG) {
@@ -221,8 +221,27 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   int lo0 = chunk > 0 ? (pos0 / chunk) * chunk : 0;
   if (window > 0) lo0 = max(lo0, pos0 - window + 1);
   __syncthreads();
-  // blockIdx.y = key split: every nsplit-th key tile (decode rows: few query rows, many keys)
-  for (int j0 = (lo0 / AT_KT + (int)blockIdx.y) * AT_KT; j0 <= last; j0 += AT_KT * nsplit) {
+  // blockIdx.y = key split: every nsplit-th key tile (decode rows: few query rows, many keys).
+  // Block-table entries are read one tile ahead (K fragments) or a phase ahead (V fragments), so
+  // no fragment load waits behind a dependent table load.
+  const int jfirst = (lo0 / AT_KT + (int)blockIdx.y) * AT_KT;
+  int nextA[2];
+#pragma unroll
+  for (int ns = 0; ns < 2; ++ns) {
+    const int key = jfirst + 16 * ns + fr;
+    nextA[ns] = key <= last ? tab[key / BS] : -1;
+  }
+  for (int j0 = jfirst; j0 <= last; j0 += AT_KT * nsplit) {
+    int blkA[2];
+#pragma unroll
+    for (int ns = 0; ns < 2; ++ns) {
+      blkA[ns] = nextA[ns];
+      const int key = j0 + AT_KT * nsplit + 16 * ns + fr;
+      nextA[ns] = key <= last ? tab[key / BS] : -1;
+    }
+    const int key8 = j0 + 8 * fq;
+    int blk8 = -1, off8 = 0;
+    if (key8 <= last) { blk8 = tab[key8 / BS]; off8 = key8 % BS; }
     // ---- A: raw scores
     for (int kb0 = 0; kb0 < KC; kb0 += 4) {      // key widths beyond 128: 128 at a time
       // 16 keys at a time: this wave's heads against their group's K fragments (B operand: key fr,
@@ -237,10 +256,8 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
           if (g != gprev) {
             gprev = g;
             const bf16* kp = nullptr;
-            if (key <= last) {
-              const int blk = tab[key / BS], off = key % BS;
-              kp = kc + (((long)blk * G + g) * BS + off) * Dk;
-            }
+            const int blk = ns ? blkA[1] : blkA[0];
+            if (blk >= 0) kp = kc + (((long)blk * G + g) * BS + key % BS) * Dk;
 #pragma unroll
             for (int kc2 = 0; kc2 < 4; ++kc2) {
               bf16x8 v = {};
@@ -258,6 +275,7 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int qr = 4 * fq + i;
+            if (qr >= nrow) continue;
             float* sp = s1 + (h * 16 + qr) * AT_SS + 16 * ns + fr;
             if (kb0 > 0) a[i] += *sp;              // partial dot products of the earlier 128 columns
             if (kb0 + 4 < KC) { *sp = a[i]; continue; }
@@ -286,7 +304,7 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
     }
     __syncthreads();
     // ---- B: head mix (fp32 MFMA) + visibility, in place
-    for (int cb = wave; cb < 2 * 16; cb += NW) {
+    for (int cb = wave; cb < 2 * nrow; cb += NW) {   // (query row, 16 keys) column blocks of the live rows
       const int qr = cb >> 1, kk = (cb & 1) * 16 + fr;
       f32x4 acc[4];
 #pragma unroll
@@ -326,8 +344,26 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
       }
     }
     __syncthreads();
+    // V fragments of this tile, requested before the softmax where the wave's heads share one kv
+    // group and the registers are there: the loads fly while phase C runs
+    constexpr bool VPRE = HPW * NDV <= 16;
+    const bool one_group = h0 < H && (h0 / rep) == ((min(h0 + HPW, H) - 1) / rep);
+    bf16x8 vpre[VPRE ? NDV : 1];
+    if constexpr (VPRE) {
+      if (one_group) {
+        const int g = h0 / rep;
+#pragma unroll
+        for (int nd = 0; nd < NDV; ++nd) {
+          const int d = 16 * nd + fr;
+          bf16x8 v = {};
+          if (blk8 >= 0 && d < Dv) v = *(const bf16x8*)(vc + (((((long)blk8 * G + g) * (BS >> 3) + (off8 >> 3)) * Dv) + d) * 8);
+          vpre[nd] = v;
+        }
+      }
+    }
     // ---- C: online softmax, a thread per (head, query) row
     for (int r = tid; r < H * 16; r += NW * 64) {
+      if ((r & 15) >= nrow) continue;            // rows past the portion's end (decode: 15 of 16)
       const float* sr = s1 + r * AT_SS;
       float mx = -INFINITY;
 #pragma unroll 8
@@ -350,9 +386,6 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
     // ---- D: O += P V; a V fragment (B operand: channel fr, keys 8 fq ..) serves every head of its group
     {
       bf16x8 pa[HPW];
-      const int key8 = j0 + 8 * fq;
-      int blk8 = -1, off8 = 0;
-      if (key8 <= last) { blk8 = tab[key8 / BS]; off8 = key8 % BS; }
 #pragma unroll
       for (int hi = 0; hi < HPW; ++hi) {
         const int h = h0 + hi;
@@ -380,9 +413,15 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
           const int g = h / rep;
           if (g != gprev) {
             gprev = g;
-            vb = bf16x8{};
-            if (blk8 >= 0 && d < Dv)
-              vb = *(const bf16x8*)(vc + (((((long)blk8 * G + g) * (BS >> 3) + (off8 >> 3)) * Dv) + d) * 8);
+            bool have = false;
+            if constexpr (VPRE) {
+              if (one_group) { vb = vpre[nd]; have = true; }
+            }
+            if (!have) {
+              vb = bf16x8{};
+              if (blk8 >= 0 && d < Dv)
+                vb = *(const bf16x8*)(vc + (((((long)blk8 * G + g) * (BS >> 3) + (off8 >> 3)) * Dv) + d) * 8);
+            }
           }
           o[hi][nd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[hi], vb, o[hi][nd], 0, 0, 0);
         }
