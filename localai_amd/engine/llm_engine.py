@@ -917,7 +917,6 @@ class LLMEngine:
         cu, qlens, dec = plan["p_cu"], plan["p_qlen"], plan["p_decode"]
         n = len(qlens)
         nc = int(n - dec.sum())          # chunks first, single-token continuations after them
-        gpu = self.device.type == "cuda"
         idx = (lambda r: self._dev(np.array(r, dtype=np.int64)) if r else None)
         if getattr(self.model, "mixed_batches", False):
             fb = ForwardBatch(tokens=self._dev(plan["p_tokens"]), pos=self._dev(plan["p_pos"]),
@@ -1509,7 +1508,11 @@ class LLMEngine:
         h["pos"][:] = torch.from_numpy(pos)
         h["slots"][:] = torch.from_numpy(slots)
         h["lens"][:] = torch.from_numpy(lens)
-        h["sslot"][:] = torch.from_numpy(self._cur_sslot)
+        ss = getattr(self, "_cur_sslot", None)   # state slots of this step's rows (_run_decode)
+        if ss is not None and len(ss) == Bp:
+            h["sslot"][:] = torch.from_numpy(ss)
+        else:
+            h["sslot"].fill_(-1)
         nb = bt.shape[1]
         h["bt"][:, :nb] = torch.from_numpy(bt)
         h["step"][0] = 0
