@@ -293,15 +293,19 @@ def test_replay_refuses_what_does_not_fit(ckpt, device):
 
 
 # --------------------------------------------------------------------------------------- generation
-@pytest.mark.parametrize("device,dtype,graphs", [("cpu", "float32", False),
-                                                 pytest.param("cuda:0", "float32", False, marks=pytest.mark.gpu),
-                                                 pytest.param("cuda:0", "bfloat16", True, marks=pytest.mark.gpu),
-                                                 pytest.param("cuda:0", "float32", True, marks=pytest.mark.gpu)])
-def test_greedy_generation_through_the_engine(ckpt, device, dtype, graphs):
+@pytest.mark.parametrize("device,dtype,graphs,name", [
+    ("cpu", "float32", False, "small"),
+    pytest.param("cuda:0", "float32", False, "small", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "bfloat16", True, "small", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "float32", True, "small", marks=pytest.mark.gpu),
+    # widths that put decode rows on the matrix-core tile kernel with key splits, inside the graphs
+    pytest.param("cuda:0", "bfloat16", True, "wide", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "bfloat16", False, "wide", marks=pytest.mark.gpu)])
+def test_greedy_generation_through_the_engine(ckpt, device, dtype, graphs, name):
     """engine.generate: scheduler-planned chunked prefill, (graph-replayed multi-step) decode with
     the device sampler, several requests at once; every emitted token is the oracle's argmax at
     its position unless the oracle's top-2 margin is within rounding."""
-    path, cfg, W = ckpt("small")
+    path, cfg, W = ckpt(name)
     eng = LLMEngine(EngineConfig(model_path=path, device=device, context_size=128, max_num_seqs=4,
                                  max_batched_tokens=24, block_size=16, use_graphs=graphs, dtype=dtype,
                                  record_tokens=True, decode_steps=4, decode_steps_wide=4))
