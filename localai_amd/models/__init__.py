@@ -7,7 +7,8 @@ from __future__ import annotations
 import importlib
 
 # architecture -> (module, class); imported lazily: some families pull in optional dependencies
-MODEL_CLASSES = {"suganex": ("localai_amd.models.suganex", "SuganexModel")}
+MODEL_CLASSES = {"suganex": ("localai_amd.models.suganex", "SuganexModel"),
+                 "dadizen": ("localai_amd.models.dadizen", "DadizenModel")}
 
 
 def model_class(arch: str):

@@ -254,22 +254,25 @@ class KVCache:
     def layered(cls, specs, num_blocks: int, block_size: int, device, dtype=torch.bfloat16,
                 state_slots: int = 0) -> "KVCache":
         """Pools for layers that differ in shape: specs[i] = (kv heads, key width, value width,
-        state shape or None).  K pages are row-major [num_blocks, heads, block_size, width]
-        (ops.kv_pages), V pages transposed per 8 keys like the other families' (ops.v_pages); layers
-        with a state shape get a pool [state_slots, *shape] beside them, indexed by the scheduler's
-        state slots.  Slots are never cleared: a kernel reads of a slot only what lies at
-        positions >= 0 of the sequence that holds it."""
+        state shape or None[, state dtype]).  K pages are row-major [num_blocks, heads, block_size,
+        width] (ops.kv_pages), V pages transposed per 8 keys like the other families' (ops.v_pages);
+        a layer without kv heads has no pages (None), one with value width 0 no V pages (its key
+        rows are also its values: latent caches).  Layers with a state shape get a pool
+        [state_slots, *shape] beside them, indexed by the scheduler's state slots, of the pool's
+        dtype unless the spec names one (recurrent state kept in fp32).  Slots are never cleared: a
+        kernel reads of a slot only what lies at positions >= 0 of the sequence that holds it."""
         kv = cls.__new__(cls)
         kv.num_blocks, kv.block_size = num_blocks, block_size
-        kv.k = [ops.kv_pages(num_blocks, g, block_size, dk, dtype, device) for g, dk, _, _ in specs]
         if block_size % 8:
             raise ValueError(f"block_size {block_size} must be a multiple of 8")
-        kv.v = [ops.v_pages(num_blocks, g, block_size, dv, dtype, device) for g, _, dv, _ in specs]
+        kv.k = [ops.kv_pages(num_blocks, sp[0], block_size, sp[1], dtype, device) if sp[0] else None for sp in specs]
+        kv.v = [ops.v_pages(num_blocks, sp[0], block_size, sp[2], dtype, device) if sp[0] and sp[2] else None
+                for sp in specs]
         kv.state_slots = state_slots
         kv.state = None
         if state_slots > 0:
-            kv.state = [torch.zeros(state_slots, *st, dtype=dtype, device=device) if st is not None else None
-                        for _, _, _, st in specs]
+            kv.state = [torch.zeros(state_slots, *sp[3], dtype=sp[4] if len(sp) > 4 else dtype, device=device)
+                        if sp[3] is not None else None for sp in specs]
         return kv
 
 

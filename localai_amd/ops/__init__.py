@@ -124,6 +124,12 @@ def lib():
             "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, I, P, P, I, P],
             "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
             "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, P],
+            "la_norm_chain": [P, I, I, P, I, LNG, I, I, F, P, P, F, P, I, I, F, P, P, P, I, P],
+            "la_glu_clamp": [P, I, LNG, I, I, I, F, F, P, I, P],
+            "la_side_gate": [P, I, LNG, I, I, I, P, P, I, I, P, I, P],
+            "la_rope_pages": [I, P, I, I, I, I, I, I, P, P, P, F, I, I, I, P, P, P, I, P],
+            "la_latent_kv": [I, P, I, I, I, P, F, P, P, P, F, I, P, I, P],
+            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
             "la_img_resample_v_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P, P, P, P, P],
         }
@@ -1837,7 +1843,8 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
              block_tables: torch.Tensor, H: int, scale: float, softcap: float = 0.0,
              slopes: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None, chunk: int = 0,
              window: int = 0, gate: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None,
-             tile_rows: int = 0, cu_q: Optional[torch.Tensor] = None, key_splits: int = 1) -> torch.Tensor:
+             tile_rows: int = 0, cu_q: Optional[torch.Tensor] = None, key_splits: int = 1,
+             v_width: int = 0) -> torch.Tensor:
     """Attention with reshaped scores over paged K ([blocks, G, BS, Dk]) and V ([blocks, G, BS / 8,
     Dv, 8], transposed per 8 keys: the operand layout of the P.V matrix instruction); one
     query row per token, row r belonging to sequence row_seq[r] (block_tables row) at position
@@ -1851,12 +1858,19 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     width % 16 and <= 128, at most 32 heads) they run on the matrix-core tile kernel, every other
     row -- fp32, odd shapes, rows after tile_rows -- on the row kernel.  key_splits > 1 deals every
     tile's keys to that many workgroups and merges their partial results in a second launch: for
-    batches of few rows with many keys each (decoding)."""
+    batches of few rows with many keys each (decoding).
+    v_cache None with v_width > 0: a key row's first v_width columns are also its value (latent
+    caches, where one stored row serves as key and value); such calls run on the row kernel."""
     T = q.shape[0]
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
-    Dv = v_cache.shape[3]
-    if v_cache.dim() != 5 or v_cache.shape[2] * 8 != BS or v_cache.shape[4] != 8:
-        raise ValueError("attn_mix: V pages must be [blocks, G, BS / 8, Dv, 8]")
+    if v_cache is None:
+        if not 0 < v_width <= Dk:
+            raise ValueError("attn_mix: without V pages v_width names the value columns of a key row")
+        Dv = int(v_width)
+    else:
+        Dv = v_cache.shape[3]
+        if v_cache.dim() != 5 or v_cache.shape[2] * 8 != BS or v_cache.shape[4] != 8:
+            raise ValueError("attn_mix: V pages must be [blocks, G, BS / 8, Dv, 8]")
     if q.shape[1] != H * Dk or H % G or row_seq.shape[0] != T or pos.shape[0] != T:
         raise ValueError("attn_mix: operand shapes do not fit")
     if not q.is_cuda:
@@ -1872,7 +1886,10 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
             tab = block_tables[int(row_seq[r])].long()
             blk, off = tab[js // BS], js % BS
             kk = k_cache[blk, :, off].float().repeat_interleave(rep, 1)     # [n, H, Dk]
-            vv = v_cache[blk, :, off // 8, :, off % 8].float().repeat_interleave(rep, 1)
+            if v_cache is None:
+                vv = kk[..., :Dv]
+            else:
+                vv = v_cache[blk, :, off // 8, :, off % 8].float().repeat_interleave(rep, 1)
             s = torch.einsum("hd,nhd->hn", qf[r], kk) * scale
             if softcap > 0:
                 s = softcap * torch.tanh(s / softcap)
@@ -1886,9 +1903,11 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
             out[r] = o
         return out.view(T, H * Dv).to(q.dtype)
     f32 = q.dtype == torch.float32
-    if q.dtype not in (torch.float32, torch.bfloat16) or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+    if (q.dtype not in (torch.float32, torch.bfloat16) or k_cache.dtype != q.dtype
+            or (v_cache is not None and v_cache.dtype != q.dtype)):
         raise ValueError("attn_mix: q and the caches share one dtype (bf16 or fp32)")
-    if not (q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and block_tables.is_contiguous()):
+    if not (q.is_contiguous() and k_cache.is_contiguous() and (v_cache is None or v_cache.is_contiguous())
+            and block_tables.is_contiguous()):
         raise ValueError("attn_mix: operands must be contiguous")
     for t in (row_seq, pos, block_tables):
         assert t.dtype == torch.int32 and t.is_cuda
@@ -1904,7 +1923,7 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
     r0 = 0
     if (tiles is not None and tile_rows > 0 and not f32 and ATTN_MIX_TILES and Dk % 32 == 0 and Dv % 16 == 0
-            and Dv <= 128 and H <= 32):
+            and Dv <= 128 and H <= 32 and v_cache is not None):
         if cu_q is None or tile_rows > T or tiles.dtype != torch.int32 or not tiles.is_contiguous():
             raise ValueError("attn_mix: tiles need cu_q and int32 [ntiles, 2]")
         ns = max(1, min(int(key_splits), 64))
@@ -1924,7 +1943,7 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     if r0 < T:
         esz = q.element_size()
         _check(lib().la_attn_mix_rows(int(f32), q.data_ptr() + r0 * H * Dk * esz, k_cache.data_ptr(),
-                                      v_cache.data_ptr(), row_seq.data_ptr() + r0 * 4, pos.data_ptr() + r0 * 4,
+                                      _ptr(v_cache), row_seq.data_ptr() + r0 * 4, pos.data_ptr() + r0 * 4,
                                       block_tables.data_ptr(), block_tables.shape[1], T - r0, H, G, Dk, Dv, BS,
                                       float(scale), float(softcap), _ptr(slopes), _ptr(talk), int(chunk), int(window),
                                       None if gate is None else gate.data_ptr() + r0 * ldg * esz, ldg,
@@ -1986,6 +2005,294 @@ def moe_pairs(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Ten
                               ids.data_ptr(), wts.data_ptr(), T, topk, D, F, E, h.data_ptr(), y.data_ptr(), _stream()),
            "la_moe_pairs")
     return y
+
+
+# ---------------------------------------------------------------------------------------
+# Layer-list designs: squashing norms, rotations into pages, latent caches, retention
+# ---------------------------------------------------------------------------------------
+
+def _branch_args(b, T: int, N: int):
+    """(pointer, is fp32, slab stride, slabs) of a [T, N] GEMM result: a Partial (fp32 split-K
+    slabs or one bf16 / fp32 matrix) or a dense contiguous tensor."""
+    t = b.t if isinstance(b, Partial) else b
+    if isinstance(b, Partial) and b.bias is not None:
+        raise ValueError("a biased partial is not taken here")
+    if t.shape[-2] != T or t.shape[-1] != N or not t.is_contiguous():
+        raise ValueError(f"operand {tuple(t.shape)} does not fit [{T}, {N}]")
+    if t.dim() == 3:
+        if t.dtype != torch.float32:
+            raise ValueError("slab sources are fp32")
+        return t.data_ptr(), 1, T * N, t.shape[0]
+    if t.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("sources are bf16 or fp32")
+    return t.data_ptr(), int(t.dtype == torch.float32), 0, 1
+
+
+def _branch_dense(b) -> torch.Tensor:
+    return b.dense() if isinstance(b, Partial) else b.float()
+
+
+NORM_NONE, NORM_DYT, NORM_RMS, NORM_CAST = 0, 1, 2, 3
+
+
+def norm_chain(res: torch.Tensor, branch=None, post: Optional[tuple] = None, pre: Optional[tuple] = None,
+               add_vec: Optional[torch.Tensor] = None, replace: bool = False,
+               out_dtype: torch.dtype = torch.bfloat16) -> Optional[torch.Tensor]:
+    """One launch per sublayer boundary of a post-normed residual stream (fp32 [T, D], updated in
+    place):  res <- (0 if replace else res) + post(branch) + add_vec, then returns pre(res).
+    post / pre:  ("dyt", alpha, w, b): tanh(alpha x) * w + b, a norm without statistics (alpha a
+    Python float, w / b fp32 [D]);  ("rms", w, eps): x / sqrt(mean(x^2) + eps) * w (post only);
+    ("cast",): res in out_dtype (pre only);  None: identity for post, no output for pre.
+    branch: a Partial or dense [T, D] tensor (None: the stream is only read).  All arithmetic fp32."""
+    T, D = res.shape
+    pm = NORM_NONE if post is None else {"dyt": NORM_DYT, "rms": NORM_RMS}[post[0]]
+    qm = NORM_NONE if pre is None else {"dyt": NORM_DYT, "cast": NORM_CAST}[pre[0]]
+    if not res.is_cuda:
+        if branch is not None:
+            y = _branch_dense(branch)
+            if pm == NORM_DYT:
+                y = torch.tanh(float(post[1]) * y) * post[2].float() + post[3].float()
+            elif pm == NORM_RMS:
+                y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + float(post[2])) * post[1].float()
+            if add_vec is not None:
+                y = y + add_vec.float()
+            if replace:
+                res.copy_(y)
+            else:
+                res += y
+        if qm == NORM_DYT:
+            return (torch.tanh(float(pre[1]) * res) * pre[2].float() + pre[3].float()).to(out_dtype)
+        return res.to(out_dtype) if qm == NORM_CAST else None
+    if res.dtype != torch.float32 or not res.is_contiguous() or out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("norm_chain: the stream is contiguous fp32; outputs are bf16 or fp32")
+    a = _branch_args(branch, T, D) if branch is not None else (None, 0, 0, 0)
+    pa, pw, pb, eps = 0.0, None, None, 0.0
+    if pm == NORM_DYT:
+        pa, pw, pb = float(post[1]), post[2], post[3]
+    elif pm == NORM_RMS:
+        pw, eps = post[1], float(post[2])
+    qa, qw_, qb = (float(pre[1]), pre[2], pre[3]) if qm == NORM_DYT else (0.0, None, None)
+    for t in (pw, pb, qw_, qb, add_vec):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != D or not t.is_contiguous()):
+            raise ValueError("norm_chain: weights are contiguous fp32 [D]")
+    out = torch.empty(T, D, dtype=out_dtype, device=res.device) if qm != NORM_NONE else None
+    _check(lib().la_norm_chain(res.data_ptr(), T, D, a[0], a[1], a[2], a[3], pm, pa, _ptr(pw), _ptr(pb), eps,
+                               _ptr(add_vec), int(replace), qm, qa, _ptr(qw_), _ptr(qb), _ptr(out),
+                               int(out_dtype == torch.float32), _stream()), "la_norm_chain")
+    return out
+
+
+def glu_clamp(src, F: int, limit: float, slope: float = 1.702, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Clamped gated unit on a gate|up projection [T, 2F]:  g = min(gate, limit), u = clamp(up,
+    -limit, limit), y = g * sigmoid(slope * g) * (u + 1).  fp32 arithmetic, [T, F] in out_dtype."""
+    t = src.t if isinstance(src, Partial) else src
+    T = t.shape[-2]
+    if t.shape[-1] != 2 * F:
+        raise ValueError("glu_clamp: the source is [T, 2F]")
+    if not t.is_cuda:
+        x = _branch_dense(src)
+        g = torch.clamp(x[:, :F], max=limit)
+        u = torch.clamp(x[:, F:], -limit, limit)
+        return (g * torch.sigmoid(slope * g) * (u + 1.0)).to(out_dtype)
+    a = _branch_args(src, T, 2 * F)
+    out = torch.empty(T, F, dtype=out_dtype, device=t.device)
+    _check(lib().la_glu_clamp(a[0], a[1], a[2], a[3], T, F, float(limit), float(slope), out.data_ptr(),
+                              int(out_dtype == torch.float32), _stream()), "la_glu_clamp")
+    return out
+
+
+def side_gate(z, tokens: torch.Tensor, table: torch.Tensor, col0: int, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """gelu_tanh(z[t]) * table[tokens[t], col0 : col0 + n] for a projection z [T, n]: a per-token
+    side embedding (bf16 [V, W] table, any column window) gated by a function of the stream."""
+    t = z.t if isinstance(z, Partial) else z
+    T, n = t.shape[-2], t.shape[-1]
+    if col0 < 0 or col0 + n > table.shape[1] or tokens.shape[0] != T:
+        raise ValueError("side_gate: the column window does not fit the table")
+    if not t.is_cuda:
+        e = table[tokens.long(), col0:col0 + n].float()
+        return (torch.nn.functional.gelu(_branch_dense(z), approximate="tanh") * e).to(out_dtype)
+    if table.dtype != torch.bfloat16 or not table.is_contiguous() or tokens.dtype != torch.int32:
+        raise ValueError("side_gate: bf16 table, int32 tokens")
+    a = _branch_args(z, T, n)
+    out = torch.empty(T, n, dtype=out_dtype, device=t.device)
+    _check(lib().la_side_gate(a[0], a[1], a[2], a[3], T, n, tokens.data_ptr(), table.data_ptr(), table.shape[1],
+                              int(col0), out.data_ptr(), int(out_dtype == torch.float32), _stream()), "la_side_gate")
+    return out
+
+
+def rot_freqs(dims: int, base: float, scaling: Optional[dict] = None, device=None) -> Tuple[torch.Tensor, float]:
+    """(angular frequencies fp32 [dims / 2], magnitude) of a rotation over `dims` dimensions:
+    f_i = base^(-2i / dims).  scaling {"factor", "original", "fast", "slow"} (YaRN): with
+    d(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor d(fast), 0), hi = min(ceil
+    d(slow), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the frequency is
+    f_i / factor * ramp_i + f_i (1 - ramp_i), and cos / sin are scaled by 0.1 ln(factor) + 1.
+    Computed in float64 on the host; the kernels form angles position * f_i in fp32."""
+    half = dims // 2
+    f = np.power(float(base), -2.0 * np.arange(half, dtype=np.float64) / dims)
+    mag = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        d_of = lambda turns: dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(base))  # noqa: E731
+        lo = max(math.floor(d_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(d_of(float(scaling["slow"]))), dims - 1)
+        ramp = np.clip((np.arange(half, dtype=np.float64) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    return torch.from_numpy(f.astype(np.float32)).to(device), float(mag)
+
+
+def _rotate_ref(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, mag: float, rot: int, off: int,
+                interleaved: bool) -> torch.Tensor:
+    """x [T, n, d] fp32 with dims [off, off + rot) of every head rotated by angle pos * freqs."""
+    ang = pos.float()[:, None] * freqs.float()[None, :]
+    c, s = (torch.cos(ang) * mag)[:, None, :], (torch.sin(ang) * mag)[:, None, :]
+    out = x.clone()
+    half = rot // 2
+    if interleaved:
+        u, v = x[..., off:off + rot:2], x[..., off + 1:off + rot:2]
+        out[..., off:off + rot:2] = u * c - v * s
+        out[..., off + 1:off + rot:2] = v * c + u * s
+    else:
+        u, v = x[..., off:off + half], x[..., off + half:off + rot]
+        out[..., off:off + half] = u * c - v * s
+        out[..., off + half:off + rot] = v * c + u * s
+    return out
+
+
+def _page_write_ref(k_cache, v_cache, slots, k, v):
+    BS = k_cache.shape[2]
+    sl = slots.long()
+    ok = sl >= 0
+    blk, off = sl[ok] // BS, sl[ok] % BS
+    if k is not None:
+        k_cache[blk, :, off] = k[ok].to(k_cache.dtype)
+    if v is not None:
+        v_cache[blk, :, off // 8, :, off % 8] = v[ok].to(v_cache.dtype)
+
+
+def rope_pages(src: torch.Tensor, H: int, Dq: int, G: int, Dk: int, Dv: int, pos: torch.Tensor,
+               slots: Optional[torch.Tensor], freqs: torch.Tensor, mag: float, rot: int, q_off: int = 0,
+               interleaved: bool = True, k_cache: Optional[torch.Tensor] = None,
+               v_cache: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotary positions on projection rows src [T, H Dq + G Dk + G Dv] (q | k | v, bf16 or fp32):
+    dims [q_off, q_off + rot) of every query head and [0, rot) of every key head are rotated by
+    the angle pos * freqs[i] (fp32), pairs (2i, 2i + 1) when interleaved, else (i, i + rot / 2),
+    cos and sin times mag; the other dims pass.  Returns q [T, H Dq]; rotated keys and the values
+    go to the paged pools (K [blocks, G, BS, Dk], V [blocks, G, BS / 8, Dv, 8]) at `slots` (-1:
+    nowhere).  G = 0: queries only."""
+    T = src.shape[0]
+    Cq, Ck, Cv = H * Dq, G * Dk, G * Dv
+    if (src.dim() != 2 or src.shape[1] != Cq + Ck + Cv or rot % 2 or q_off + rot > Dq or (G and rot > Dk)
+            or freqs.numel() != rot // 2 or pos.shape[0] != T):
+        raise ValueError("rope_pages: operand shapes do not fit")
+    if G and (k_cache is None or v_cache is None or slots is None or tuple(k_cache.shape[1:]) != (G, k_cache.shape[2], Dk)
+              or tuple(v_cache.shape[1:]) != (G, k_cache.shape[2] // 8, Dv, 8)):
+        raise ValueError("rope_pages: pools do not fit the key / value widths")
+    if not src.is_cuda:
+        x = src.float()
+        q = _rotate_ref(x[:, :Cq].reshape(T, H, Dq), pos, freqs, mag, rot, q_off, interleaved)
+        if G:
+            k = _rotate_ref(x[:, Cq:Cq + Ck].reshape(T, G, Dk), pos, freqs, mag, rot, 0, interleaved)
+            _page_write_ref(k_cache, v_cache, slots, k, x[:, Cq + Ck:].reshape(T, G, Dv))
+        return q.reshape(T, Cq).to(src.dtype)
+    f32 = src.dtype == torch.float32
+    if src.dtype not in (torch.float32, torch.bfloat16) or not src.is_contiguous():
+        raise ValueError("rope_pages: contiguous bf16 or fp32 rows")
+    if G and (k_cache.dtype != src.dtype or v_cache.dtype != src.dtype):
+        raise ValueError("rope_pages: pools share the rows' dtype")
+    assert pos.dtype == torch.int32 and freqs.dtype == torch.float32 and freqs.is_contiguous()
+    assert slots is None or (slots.dtype == torch.int32 and slots.shape[0] == T)
+    q = torch.empty(T, Cq, dtype=src.dtype, device=src.device)
+    _check(lib().la_rope_pages(int(f32), src.data_ptr(), T, H, Dq, G, Dk, Dv, pos.data_ptr(), _ptr(slots),
+                               freqs.data_ptr(), float(mag), rot, q_off, int(interleaved), q.data_ptr(),
+                               _ptr(k_cache), _ptr(v_cache), k_cache.shape[2] if G else 0, _stream()), "la_rope_pages")
+    return q
+
+
+def latent_kv(src: torch.Tensor, rank: int, norm_w: torch.Tensor, eps: float, pos: torch.Tensor, slots: torch.Tensor,
+              freqs: torch.Tensor, mag: float, k_cache: torch.Tensor, interleaved: bool = True) -> None:
+    """Latent key/value rows into a one-head pool [blocks, 1, BS, rank + rot]: of a down-projection
+    row src[t] = [c (rank) | r (rot)] the latent part is RMS-normed (c / sqrt(mean c^2 + eps) *
+    norm_w, fp32) and the rest rotated by pos[t] * freqs; the stored row [norm c | rot r] is key
+    and value at once (attn_mix, v_width = rank)."""
+    T, W = src.shape
+    rot = W - rank
+    if (rank <= 0 or rot < 0 or rot % 2 or freqs.numel() != rot // 2 or norm_w.numel() != rank
+            or k_cache.shape[1] != 1 or k_cache.shape[3] != W or pos.shape[0] != T or slots.shape[0] != T):
+        raise ValueError("latent_kv: operand shapes do not fit")
+    if not src.is_cuda:
+        x = src.float()
+        c = x[:, :rank]
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+        r = _rotate_ref(x[:, rank:].reshape(T, 1, rot), pos, freqs, mag, rot, 0, interleaved).reshape(T, rot)
+        _page_write_ref(k_cache, None, slots, torch.cat([c, r], -1).reshape(T, 1, W), None)
+        return
+    if src.dtype not in (torch.float32, torch.bfloat16) or not src.is_contiguous() or k_cache.dtype != src.dtype:
+        raise ValueError("latent_kv: contiguous bf16 or fp32 rows, pool of the same dtype")
+    assert pos.dtype == torch.int32 and slots.dtype == torch.int32 and freqs.dtype == torch.float32
+    assert norm_w.dtype == torch.float32 and norm_w.is_contiguous()
+    _check(lib().la_latent_kv(int(src.dtype == torch.float32), src.data_ptr(), T, rank, rot, norm_w.data_ptr(),
+                              float(eps), pos.data_ptr(), slots.data_ptr(), freqs.data_ptr(), float(mag),
+                              int(interleaved), k_cache.data_ptr(), k_cache.shape[2], _stream()), "la_latent_kv")
+
+
+def retention_state(slots: int, H: int, Dk: int, Dv: int, device=None) -> torch.Tensor:
+    """State pool of ops.retention: fp32 [slots, H, Dv, Dk], every head's Dk x Dv state stored
+    value-column major (a column's Dk entries contiguous: the kernel's threads own columns)."""
+    return torch.zeros(slots, H, Dv, Dk, dtype=torch.float32, device=device)
+
+
+def retention(src: torch.Tensor, H: int, Dk: int, Dv: int, pos: torch.Tensor, cu_q: torch.Tensor,
+              sslots: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, freqs: torch.Tensor, rot: int,
+              eps: float, mag: float = 1.0) -> torch.Tensor:
+    """Decayed linear attention over projection rows src [T, 2 H Dk + 2 H Dv] (q | k | v | gate):
+    q and k rotated on their first `rot` dims (pairs (i, i + rot / 2), angle pos * freqs[i]), k
+    times Dk^-1/2; per head S <- decay_h S + k v^T, o = S^T q (no softmax, no denominator); o
+    divided by its root mean square over the head (eps), times silu(gate).  Rows of a sequence
+    portion are consecutive (cu_q [nseq + 1]); its state lives in state[sslots[seq]] (fp32,
+    retention_state), is taken as zero when the portion starts at position 0 and advanced to the
+    portion's end.  Rotation, state, outputs and the norm are fp32.  Returns [T, H Dv] in src's dtype."""
+    T = src.shape[0]
+    nseq = cu_q.shape[0] - 1
+    Cq, Cv = H * Dk, H * Dv
+    if (src.dim() != 2 or src.shape[1] != 2 * Cq + 2 * Cv or tuple(state.shape[1:]) != (H, Dv, Dk) or decay.numel() != H
+            or rot % 2 or rot > Dk or freqs.numel() != rot // 2 or sslots.shape[0] != nseq or pos.shape[0] != T):
+        raise ValueError("retention: operand shapes do not fit")
+    if not src.is_cuda:
+        x = src.float()
+        q = _rotate_ref(x[:, :Cq].reshape(T, H, Dk), pos, freqs, mag, rot, 0, False)
+        k = _rotate_ref(x[:, Cq:2 * Cq].reshape(T, H, Dk), pos, freqs, mag, rot, 0, False) * Dk ** -0.5
+        v = x[:, 2 * Cq:2 * Cq + Cv].reshape(T, H, Dv)
+        g = x[:, 2 * Cq + Cv:].reshape(T, H, Dv)
+        o = torch.zeros(T, H, Dv)
+        cu = cu_q.tolist()
+        d = decay.float().view(H, 1, 1)
+        for s in range(nseq):
+            a, b = cu[s], cu[s + 1]
+            if b <= a:
+                continue
+            ss = int(sslots[s])
+            S = torch.zeros(H, Dk, Dv) if int(pos[a]) == 0 else state[ss].float().transpose(1, 2).clone()
+            for t in range(a, b):
+                S = d * S + k[t].unsqueeze(2) * v[t].unsqueeze(1)
+                o[t] = torch.einsum("hkv,hk->hv", S, q[t])
+            state[ss] = S.transpose(1, 2)
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        return (o * torch.nn.functional.silu(g)).reshape(T, Cv).to(src.dtype)
+    if src.dtype not in (torch.float32, torch.bfloat16) or not src.is_contiguous():
+        raise ValueError("retention: contiguous bf16 or fp32 rows")
+    if state.dtype != torch.float32 or not state.is_contiguous():
+        raise ValueError("retention: the state pool is contiguous fp32")
+    for t in (pos, cu_q, sslots):
+        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+    assert decay.dtype == torch.float32 and freqs.dtype == torch.float32
+    o = torch.empty(T, Cv, dtype=torch.float32, device=src.device)
+    out = torch.empty(T, Cv, dtype=src.dtype, device=src.device)
+    _check(lib().la_retention(int(src.dtype == torch.float32), src.data_ptr(), T, nseq, H, Dk, Dv, pos.data_ptr(),
+                              cu_q.data_ptr(), sslots.data_ptr(), state.data_ptr(), state.shape[0], decay.data_ptr(),
+                              freqs.data_ptr(), float(mag), rot, float(eps), o.data_ptr(), out.data_ptr(), _stream()),
+           "la_retention")
+    return out
 
 
 # ---------------------------------------------------------------------------------------
