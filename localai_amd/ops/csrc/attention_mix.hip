@@ -11,7 +11,8 @@
 // online-softmax step per head (a wave per head, a lane per key) and accumulates P.V with threads
 // spread over (head, value channel).  Query rows are independent (row -> sequence, position), so a
 // launch takes prompt portions and single decoded tokens alike.  K and V rows of key and value
-// width Dk / Dv may differ.  Scores, softmax and the accumulators are fp32; q, K, V, gate logits
+// width Dk / Dv may differ; the row kernel also takes pools without V pages, where the first Dv
+// columns of a key row are its value.  Scores, softmax and the accumulators are fp32; q, K, V, gate logits
 // and the output are the activation type (bf16 or fp32).
 #include "common.h"
 
@@ -132,9 +133,16 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
       if (o < HV) {
         const int h = o / Dv, d = o - h * Dv, g = h / rep;
         float a = acc[e] * alpha[h];
-        for (int jj = 0; jj < nk; ++jj) {
-          const int j = j0 + jj, blk = tab[j / BS], off = j % BS;
-          a = fmaf(s2[h * AM_KT + jj], (float)vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)], a);
+        if (vc) {
+          for (int jj = 0; jj < nk; ++jj) {
+            const int j = j0 + jj, blk = tab[j / BS], off = j % BS;
+            a = fmaf(s2[h * AM_KT + jj], (float)vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)], a);
+          }
+        } else {   // no V pages: a key row's first Dv columns are its value (latent caches)
+          for (int jj = 0; jj < nk; ++jj) {
+            const int j = j0 + jj, blk = tab[j / BS], off = j % BS;
+            a = fmaf(s2[h * AM_KT + jj], (float)kc[(((long)blk * G + g) * BS + off) * Dk + d], a);
+          }
         }
         acc[e] = a;
       }

@@ -1,0 +1,210 @@
+// Sublayer boundaries of a post-normed fp32 residual stream, and the small elementwise steps of
+// layer-list designs that sit between two library GEMMs.
+//
+//   norm_chain:  res <- (replace ? 0 : res) + post(branch) + add_vec;  out = pre(res)
+//       post:  none | dyt: tanh(alpha y) * w + b | rms: y / sqrt(mean(y^2) + eps) * w
+//       pre:   none | dyt | cast (the stream itself in the output type)
+//     one launch where a pre-normed stream has "add + norm": the branch's own norm, the residual
+//     add and the next sublayer's input norm.  A workgroup per row; the rms variant reads the
+//     branch row twice (second time from cache) instead of holding it in registers, so any width runs.
+//   glu_clamp:   g = min(gate, limit), u = clamp(up, -limit, limit), y = g sigmoid(slope g) (u + 1)
+//   side_gate:   gelu_tanh(z[t][c]) * table[tok[t]][col0 + c]
+//
+// Sources are GEMM results as the framework hands them on: fp32 split-K slabs [S][T][N] (summed
+// here), or one bf16 / fp32 matrix.  All arithmetic is fp32; outputs bf16 or fp32.
+#include "common.h"
+
+namespace la {
+
+struct RowSrc {
+  const void* p;
+  int f32;
+  long slab;
+  int S;
+};
+
+LA_DEV float src_at(const RowSrc& s, long idx) {
+  if (s.f32) {
+    const float* f = (const float*)s.p;
+    float a = f[idx];
+    for (int k = 1; k < s.S; ++k) a += f[idx + k * s.slab];
+    return a;
+  }
+  return (float)((const bf16*)s.p)[idx];
+}
+
+LA_DEV void put(void* out, int out_f32, long idx, float v) {
+  if (out_f32) ((float*)out)[idx] = v;
+  else ((bf16*)out)[idx] = (bf16)v;
+}
+
+enum { NC_NONE = 0, NC_DYT = 1, NC_RMS = 2, NC_CAST = 3 };
+constexpr int NC_NT = 256;
+
+__global__ __launch_bounds__(NC_NT) void norm_chain_kernel(float* __restrict__ res, int D, RowSrc src, int has_src,
+                                                           int post, float pa, const float* __restrict__ pw,
+                                                           const float* __restrict__ pb, float eps,
+                                                           const float* __restrict__ addv, int replace, int pre,
+                                                           float qa, const float* __restrict__ qw,
+                                                           const float* __restrict__ qb, void* __restrict__ out,
+                                                           int out_f32) {
+  __shared__ float red[NC_NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const long base = (long)t * D;
+  float inv = 1.f;
+  if (has_src && post == NC_RMS) {
+    float ss = 0.f;
+    for (int c = tid; c < D; c += NC_NT) {
+      const float y = src_at(src, base + c);
+      ss = fmaf(y, y, ss);
+    }
+    ss = block_sum<NC_NT>(ss, red);
+    inv = 1.f / sqrtf(ss / (float)D + eps);
+  }
+  for (int c = tid; c < D; c += NC_NT) {
+    float x = res[base + c];
+    if (has_src) {
+      float y = src_at(src, base + c);
+      if (post == NC_DYT) y = fmaf(tanhf(pa * y), pw[c], pb[c]);
+      else if (post == NC_RMS) y = y * inv * pw[c];
+      if (addv) y += addv[c];
+      x = replace ? y : x + y;
+      res[base + c] = x;
+    }
+    if (pre == NC_DYT) put(out, out_f32, base + c, fmaf(tanhf(qa * x), qw[c], qb[c]));
+    else if (pre == NC_CAST) put(out, out_f32, base + c, x);
+  }
+}
+
+// widths that are a multiple of 4 with one-matrix sources: 4 columns per thread, 16-byte accesses to the stream
+__global__ __launch_bounds__(NC_NT) void norm_chain4_kernel(float* __restrict__ res, int D, const void* __restrict__ sp,
+                                                            int src_f32, int has_src, int post, float pa,
+                                                            const float* __restrict__ pw, const float* __restrict__ pb,
+                                                            float eps, const float* __restrict__ addv, int replace,
+                                                            int pre, float qa, const float* __restrict__ qw,
+                                                            const float* __restrict__ qb, void* __restrict__ out,
+                                                            int out_f32) {
+  __shared__ float red[NC_NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const long base = (long)t * D;
+  auto load = [&](int c, float* y) {
+    if (src_f32) {
+      const float4 v = *(const float4*)((const float*)sp + base + c);
+      y[0] = v.x; y[1] = v.y; y[2] = v.z; y[3] = v.w;
+    } else {
+      const bf16x4 v = *(const bf16x4*)((const bf16*)sp + base + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) y[j] = (float)v[j];
+    }
+  };
+  float inv = 1.f;
+  if (has_src && post == NC_RMS) {
+    float ss = 0.f;
+    for (int c = tid * 4; c < D; c += NC_NT * 4) {
+      float y[4];
+      load(c, y);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ss = fmaf(y[j], y[j], ss);
+    }
+    ss = block_sum<NC_NT>(ss, red);
+    inv = 1.f / sqrtf(ss / (float)D + eps);
+  }
+  for (int c = tid * 4; c < D; c += NC_NT * 4) {
+    const float4 xv = *(const float4*)(res + base + c);
+    float x[4] = {xv.x, xv.y, xv.z, xv.w};
+    if (has_src) {
+      float y[4];
+      load(c, y);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (post == NC_DYT) y[j] = fmaf(tanhf(pa * y[j]), pw[c + j], pb[c + j]);
+        else if (post == NC_RMS) y[j] = y[j] * inv * pw[c + j];
+        if (addv) y[j] += addv[c + j];
+        x[j] = replace ? y[j] : x[j] + y[j];
+      }
+      *(float4*)(res + base + c) = make_float4(x[0], x[1], x[2], x[3]);
+    }
+    if (pre != NC_NONE) {
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = pre == NC_DYT ? fmaf(tanhf(qa * x[j]), qw[c + j], qb[c + j]) : x[j];
+      if (out_f32) *(float4*)((float*)out + base + c) = make_float4(o[0], o[1], o[2], o[3]);
+      else {
+        bf16x4 ob = {(bf16)o[0], (bf16)o[1], (bf16)o[2], (bf16)o[3]};
+        *(bf16x4*)((bf16*)out + base + c) = ob;
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void glu_clamp_kernel(RowSrc src, int F, long total, float limit, float slope,
+                                                        void* __restrict__ out, int out_f32) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long t = e / F;
+  const int c = (int)(e - t * F);
+  const float g = fminf(src_at(src, t * 2 * F + c), limit);
+  const float u = fminf(fmaxf(src_at(src, t * 2 * F + F + c), -limit), limit);
+  put(out, out_f32, e, g / (1.f + expf(-slope * g)) * (u + 1.f));
+}
+
+LA_DEV float gelu_tanh_f(float x) { return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x))); }
+
+__global__ __launch_bounds__(256) void side_gate_kernel(RowSrc src, int n, long total, const int* __restrict__ tok,
+                                                        const bf16* __restrict__ table, int ldt, int col0,
+                                                        void* __restrict__ out, int out_f32) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long t = e / n;
+  const int c = (int)(e - t * n);
+  const float emb = (float)table[(long)tok[t] * ldt + col0 + c];
+  put(out, out_f32, e, gelu_tanh_f(src_at(src, e)) * emb);
+}
+
+}  // namespace la
+
+extern "C" int la_norm_chain(void* res, int T, int D, const void* sp, int src_f32, long slab, int S, int post, float pa,
+                             const void* pw, const void* pb, float eps, const void* addv, int replace, int pre, float qa,
+                             const void* qw, const void* qb, void* out, int out_f32, void* stream) {
+  using namespace la;
+  if (T <= 0 || D <= 0 || !res) return -1;
+  if (post == NC_DYT && (!pw || !pb)) return -2;
+  if (post == NC_RMS && !pw) return -2;
+  if (pre == NC_DYT && (!qw || !qb)) return -2;
+  if (pre != NC_NONE && !out) return -3;
+  const int has = sp != nullptr;
+  if (has && src_f32 && S < 1) return -4;
+  if ((D & 3) == 0 && (!has || S <= 1)) {
+    hipLaunchKernelGGL(norm_chain4_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, (float*)res, D, sp, src_f32, has,
+                       post, pa, (const float*)pw, (const float*)pb, eps, (const float*)addv, replace, pre, qa,
+                       (const float*)qw, (const float*)qb, out, out_f32);
+    return (int)hipGetLastError();
+  }
+  RowSrc s{sp, src_f32, slab, S};
+  hipLaunchKernelGGL(norm_chain_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, (float*)res, D, s, has, post, pa,
+                     (const float*)pw, (const float*)pb, eps, (const float*)addv, replace, pre, qa, (const float*)qw,
+                     (const float*)qb, out, out_f32);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_glu_clamp(const void* sp, int src_f32, long slab, int S, int T, int F, float limit, float slope,
+                            void* out, int out_f32, void* stream) {
+  using namespace la;
+  if (T <= 0 || F <= 0 || !sp || !out) return -1;
+  RowSrc s{sp, src_f32, slab, S};
+  const long total = (long)T * F;
+  hipLaunchKernelGGL(glu_clamp_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, s, F,
+                     total, limit, slope, out, out_f32);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_side_gate(const void* sp, int src_f32, long slab, int S, int T, int n, const void* tok,
+                            const void* table, int ldt, int col0, void* out, int out_f32, void* stream) {
+  using namespace la;
+  if (T <= 0 || n <= 0 || !sp || !out || !tok || !table || col0 < 0 || col0 + n > ldt) return -1;
+  RowSrc s{sp, src_f32, slab, S};
+  const long total = (long)T * n;
+  hipLaunchKernelGGL(side_gate_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, s, n,
+                     total, (const int*)tok, (const bf16*)table, ldt, col0, out, out_f32);
+  return (int)hipGetLastError();
+}

@@ -1,0 +1,146 @@
+// Rotary positions on projection rows and the append of keys / values into the paged pools, for
+// designs whose key and value widths differ, whose rotation covers part of a head at an offset, and
+// whose frequencies are a table (YaRN-scaled or plain) rather than one base.
+//
+//   rope_pages:  row [q (H x Dq) | k (G x Dk) | v (G x Dv)];  dims [q_off, q_off + rot) of every
+//                query head and [0, rot) of every key head are rotated, pair (2i, 2i + 1)
+//                (interleaved) or (i, i + rot / 2):  (u, v) -> (u c - v s, v c + u s), angle
+//                pos * freq[i] formed and evaluated in fp32, c and s times `mag`.
+//                K rows go to [blocks][G][BS][Dk], V to [blocks][G][BS / 8][Dv][8].
+//   latent_kv:   row [c (rank) | r (rot)]:  c / sqrt(mean c^2 + eps) * w and the rotated r are stored
+//                as ONE row of a one-head K pool, [blocks][1][BS][rank + rot]: key and value at once.
+//
+// A workgroup per token; the token's cos / sin are computed once into LDS.
+#include "common.h"
+
+namespace la {
+
+constexpr int RP_NT = 256;
+
+// rotated value of dim d (relative to the start of the rotated span) of a head whose span starts at x
+template <typename AT>
+LA_DEV float rot_dim(const AT* __restrict__ x, int d, int rot, int interleaved, const float* __restrict__ cs) {
+  const int half = rot >> 1;
+  int i, first;
+  float u, v;
+  if (interleaved) {
+    i = d >> 1;
+    first = !(d & 1);
+    u = (float)x[d & ~1];
+    v = (float)x[d | 1];
+  } else {
+    first = d < half;
+    i = first ? d : d - half;
+    u = (float)x[i];
+    v = (float)x[i + half];
+  }
+  const float c = cs[2 * i], s = cs[2 * i + 1];
+  return first ? u * c - v * s : v * c + u * s;
+}
+
+LA_DEV void fill_cos_sin(float* cs, int rot, int p, const float* __restrict__ freqs, float mag) {
+  for (int i = threadIdx.x; i < (rot >> 1); i += blockDim.x) {
+    const float a = (float)p * freqs[i];
+    cs[2 * i] = cosf(a) * mag;
+    cs[2 * i + 1] = sinf(a) * mag;
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(RP_NT) void rope_pages_kernel(const AT* __restrict__ src, int H, int Dq, int G, int Dk, int Dv,
+                                                           const int* __restrict__ pos, const int* __restrict__ slots,
+                                                           const float* __restrict__ freqs, float mag, int rot, int q_off,
+                                                           int interleaved, AT* __restrict__ q_out, AT* __restrict__ kc,
+                                                           AT* __restrict__ vc, int BS) {
+  extern __shared__ float cs[];          // [rot / 2][2]
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int Cq = H * Dq, Ck = G * Dk, Cv = G * Dv;
+  const AT* row = src + (long)t * (Cq + Ck + Cv);
+  fill_cos_sin(cs, rot, pos[t], freqs, mag);
+  __syncthreads();
+  for (int e = tid; e < Cq; e += RP_NT) {
+    const int h = e / Dq, d = e - h * Dq;
+    float o;
+    if (d >= q_off && d < q_off + rot) o = rot_dim<AT>(row + h * Dq + q_off, d - q_off, rot, interleaved, cs);
+    else o = (float)row[e];
+    q_out[(long)t * Cq + e] = (AT)o;
+  }
+  if (!G) return;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const int blk = slot / BS, off = slot - blk * BS;
+  for (int e = tid; e < Ck; e += RP_NT) {
+    const int g = e / Dk, d = e - g * Dk;
+    const float o = d < rot ? rot_dim<AT>(row + Cq + g * Dk, d, rot, interleaved, cs) : (float)row[Cq + e];
+    kc[(((long)blk * G + g) * BS + off) * Dk + d] = (AT)o;
+  }
+  for (int e = tid; e < Cv; e += RP_NT) {
+    const int g = e / Dv, d = e - g * Dv;
+    vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)] = row[Cq + Ck + e];
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(RP_NT) void latent_kv_kernel(const AT* __restrict__ src, int rank, int rot,
+                                                          const float* __restrict__ w, float eps,
+                                                          const int* __restrict__ pos, const int* __restrict__ slots,
+                                                          const float* __restrict__ freqs, float mag, int interleaved,
+                                                          AT* __restrict__ kc, int BS) {
+  extern __shared__ float cs[];          // [rot / 2][2]
+  __shared__ float red[RP_NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int slot = slots[t];
+  if (slot < 0) return;                  // uniform over the workgroup
+  const int W = rank + rot;
+  const AT* row = src + (long)t * W;
+  fill_cos_sin(cs, rot, pos[t], freqs, mag);
+  float ss = 0.f;
+  for (int c = tid; c < rank; c += RP_NT) {
+    const float x = (float)row[c];
+    ss = fmaf(x, x, ss);
+  }
+  ss = block_sum<RP_NT>(ss, red);        // its barriers also publish cs
+  const float inv = 1.f / sqrtf(ss / (float)rank + eps);
+  AT* dst = kc + (long)slot * W;         // one head: page row = slot
+  for (int c = tid; c < rank; c += RP_NT) dst[c] = (AT)((float)row[c] * inv * w[c]);
+  for (int d = tid; d < rot; d += RP_NT) dst[rank + d] = (AT)rot_dim<AT>(row + rank, d, rot, interleaved, cs);
+  (void)BS;
+}
+
+}  // namespace la
+
+extern "C" int la_rope_pages(int f32, const void* src, int T, int H, int Dq, int G, int Dk, int Dv, const void* pos,
+                             const void* slots, const void* freqs, float mag, int rot, int q_off, int interleaved,
+                             void* q_out, void* kc, void* vc, int BS, void* stream) {
+  using namespace la;
+  if (T <= 0 || H <= 0 || Dq <= 0 || G < 0 || (rot & 1) || rot < 0 || q_off < 0 || q_off + rot > Dq) return -1;
+  if (G && (rot > Dk || !kc || !vc || !slots || BS <= 0 || (BS & 7))) return -2;
+  if (!src || !pos || !freqs || !q_out) return -3;
+  const size_t shm = (size_t)(rot > 0 ? rot : 2) * sizeof(float);
+  if (f32)
+    hipLaunchKernelGGL(rope_pages_kernel<float>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const float*)src, H, Dq,
+                       G, Dk, Dv, (const int*)pos, (const int*)slots, (const float*)freqs, mag, rot, q_off, interleaved,
+                       (float*)q_out, (float*)kc, (float*)vc, BS);
+  else
+    hipLaunchKernelGGL(rope_pages_kernel<bf16>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const bf16*)src, H, Dq, G,
+                       Dk, Dv, (const int*)pos, (const int*)slots, (const float*)freqs, mag, rot, q_off, interleaved,
+                       (bf16*)q_out, (bf16*)kc, (bf16*)vc, BS);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_latent_kv(int f32, const void* src, int T, int rank, int rot, const void* w, float eps, const void* pos,
+                            const void* slots, const void* freqs, float mag, int interleaved, void* kc, int BS,
+                            void* stream) {
+  using namespace la;
+  if (T <= 0 || rank <= 0 || rot < 0 || (rot & 1) || !src || !w || !pos || !slots || !freqs || !kc) return -1;
+  const size_t shm = (size_t)(rot > 0 ? rot : 2) * sizeof(float);
+  if (f32)
+    hipLaunchKernelGGL(latent_kv_kernel<float>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const float*)src, rank,
+                       rot, (const float*)w, eps, (const int*)pos, (const int*)slots, (const float*)freqs, mag, interleaved,
+                       (float*)kc, BS);
+  else
+    hipLaunchKernelGGL(latent_kv_kernel<bf16>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const bf16*)src, rank, rot,
+                       (const float*)w, eps, (const int*)pos, (const int*)slots,
+                       (const float*)freqs, mag, interleaved, (bf16*)kc, BS);
+  return (int)hipGetLastError();
+}
