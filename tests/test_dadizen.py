@@ -71,7 +71,7 @@ CONFIGS = {
                  ff(reten(heads=2, dim=6, vdim=10, decay=(0.95, 0.999), dims=6), 40),
                  ff(attn(heads=2, kv=1, dim=12, vdim=4, window=1000, dims=6), 40)]},
     "plain": {"vocab": 40, "width": 24, "norm": {"eps": 1e-5}, "layers": [
-        ff(attn(heads=2, kv=2, dim=6, vdim=6, window=7, dims=6), 20), ff(reten(heads=2, dim=4, vdim=4), 20),
+        ff(attn(heads=2, kv=2, dim=6, vdim=6, window=7, dims=6), 20), ff(reten(heads=2, dim=4, vdim=4, dims=4), 20),
         ff(latent(heads=2, dim=4, rot_dim=4, vdim=4, q_rank=6, kv_rank=6), 20)]},
     # widths the GPU's specialised paths take: key width % 32 and value width % 16 (matrix-core
     # attention tiles), GEMM depths % 256 (skinny GEMMs), retention rows over several registers a lane
