@@ -1354,3 +1354,78 @@ def write_suganex(out_dir: str, width: int = 256, n_layer: int = 2, heads: int =
         json.dump(cfg, f)
     save_file(W, os.path.join(out_dir, "model.safetensors"))
     return out_dir
+
+
+def write_dadizen(out_dir: str, width: int = 256, kinds=("attention", "latent_attention", "retention"), heads: int = 4,
+                  kv_heads: int = 2, dim: int = 64, vdim: int = 64, window: int = 256, rot_dim: int = 32,
+                  q_rank: int = 128, kv_rank: int = 64, ff: int = 1024, side_dim: int = 32, loop=None,
+                  vocab: int = 32000, seed: int = 0) -> str:
+    """Random-init Dadizen checkpoint directory (config.json + model.safetensors, bf16): one layer
+    per entry of `kinds` (the mixer types), all of the given sizes, every layer with a clamped gated
+    feed-forward of width `ff` and a token side input of `side_dim` columns (0: none); loop =
+    (start, stop, times) or None.  Benchmarks and smoke runs; the weights mean nothing."""
+    import json
+
+    import torch
+    from safetensors.torch import save_file
+    os.makedirs(out_dir, exist_ok=True)
+    g = torch.Generator().manual_seed(seed)
+    D, n = width, len(kinds)
+
+    def rnd(*shape, s):
+        return (torch.randn(*shape, generator=g, dtype=torch.float32) * s).to(torch.bfloat16)
+
+    def lin(a, b):
+        return rnd(a, b, s=b ** -0.5)
+
+    yarn = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    W = {"embed": rnd(vocab, D, s=1.0), "head": lin(vocab, D)}
+
+    def norm(name):
+        W[name], W[name + ".b"] = (1.0 + rnd(D, s=0.05).float()).to(torch.bfloat16), rnd(D, s=0.02)
+        W[name + ".alpha"] = torch.tensor(0.7).to(torch.bfloat16)
+
+    norm("final.norm")
+    if side_dim:
+        W["side.embed"] = rnd(vocab, n * side_dim, s=1.0)
+    layers = []
+    for i, kind in enumerate(kinds):
+        p = f"l{i}."
+        for nm in ("norm1", "norm1b", "norm2", "norm2b"):
+            norm(p + nm)
+        if kind == "attention":
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                 "mask": {"size": window}, "rot": {"dims": dim, "base": 10000.0, "scaling": yarn}}
+            W[p + "mix.q"], W[p + "mix.k"], W[p + "mix.v"] = lin(heads * dim, D), lin(kv_heads * dim, D), lin(kv_heads * vdim, D)
+        elif kind == "latent_attention":
+            m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+                 "scale": (dim + rot_dim) ** -0.5, "rot": {"dims": rot_dim, "base": 10000.0, "scaling": yarn}}
+            W[p + "mix.dq"], W[p + "mix.dq.norm"] = lin(q_rank, D), (1.0 + rnd(q_rank, s=0.05).float()).to(torch.bfloat16)
+            W[p + "mix.uq"] = lin(heads * (dim + rot_dim), q_rank)
+            W[p + "mix.dkv"] = lin(kv_rank + rot_dim, D)
+            W[p + "mix.dkv.norm"] = (1.0 + rnd(kv_rank, s=0.05).float()).to(torch.bfloat16)
+            W[p + "mix.uk"], W[p + "mix.uv"], W[p + "mix.g"] = lin(heads * dim, kv_rank), lin(heads * vdim, kv_rank), lin(heads, D)
+        elif kind == "retention":
+            m = {"heads": heads, "dim": dim, "vdim": vdim, "decay": [1.0 - 2.0 ** (-5 - h % 4) for h in range(heads)],
+                 "rot": {"dims": dim, "base": 10000.0}}
+            W[p + "mix.q"], W[p + "mix.k"] = lin(heads * dim, D), lin(heads * dim, D)
+            W[p + "mix.v"], W[p + "mix.g"] = lin(heads * vdim, D), lin(heads * vdim, D)
+        else:
+            raise ValueError(f"unknown mixer kind {kind!r}")
+        W[p + "mix.o"] = lin(D, heads * vdim)
+        W[p + "mlp.gate"], W[p + "mlp.up"], W[p + "mlp.down"] = lin(ff, D), lin(ff, D), lin(D, ff)
+        if side_dim:
+            W[p + "side.gate"], W[p + "side.proj"], W[p + "side.norm"] = lin(side_dim, D), lin(D, side_dim), rnd(D, s=0.1)
+        layers.append({"type": kind, "mixer": m, "mlp": {"kind": "dense", "ff": ff, "limit": 7.0}})
+    cfg = {"architecture": "Dadizen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": layers,
+           "logit_softcap": 50.0}
+    if side_dim:
+        cfg["token_side"] = {"dim": side_dim}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+        W["loop.in"] = torch.cat([torch.eye(D) * 0.7, torch.eye(D) * 0.3], 1).to(torch.bfloat16)
+        W["loop.step"] = rnd(loop[2], D, s=0.1)
+    with open(os.path.join(out_dir, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file(W, os.path.join(out_dir, "model.safetensors"))
+    return out_dir

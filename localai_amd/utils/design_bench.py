@@ -1,9 +1,10 @@
 """Prefill and decode throughput of a model design beside the closest decoder family at equal
 layer sizes (bench.py --design-compare): random weights, bf16, one GPU.
 
-For each size two pairs of two-layer models are built -- dense feed-forwards (Suganex vs a llama
-checkpoint) and routed experts (Suganex vs a Mixtral-style checkpoint), both stored as dense bf16
-weights so every GEMM takes the same library path -- and each is timed through its engine's own
+For each size two-layer models are built -- Suganex: dense feed-forwards (beside a llama
+checkpoint) and routed experts (beside a Mixtral-style checkpoint); Dadizen: one model per mixer
+kind (windowed attention, latent attention, retention) beside the llama checkpoint -- all stored as
+dense bf16 weights so every GEMM takes the same library path, and each is timed through its engine's own
 batch construction (native scheduler, paged KV pool, state slots) and `model.forward`:
   prefill: `n_seq` prompts of `prompt` tokens in one batch, tokens/s;
   decode:  `batch` sequences holding `context` tokens each, one token per sequence and step, tokens/s
@@ -28,6 +29,43 @@ SIZES = {
     "4k": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, experts=8, top=2, eff=3584, chunk=1024),
 }
 VOCAB = 32000
+
+
+def _llama(size: str, cache: str, moe: bool = False) -> str:
+    from ..models import synth
+    s = SIZES[size]
+    kind = "moe" if moe else "dense"
+    g = os.path.join(cache, f"llama-{size}-{kind}-f16.gguf")
+    if not os.path.exists(g):
+        pre = synth.Preset(n_layer=2, n_embd=s["width"], n_head=s["heads"], n_head_kv=s["kv"], head_dim=s["dim"],
+                           n_ff=s["eff"] if moe else s["ff"], n_vocab=VOCAB, ctx=8192, qtype="F16",
+                           n_expert=s["experts"] if moe else 0, n_expert_used=s["top"] if moe else 0,
+                           tokenizer="mistral", name=f"llama-{size}-{kind}")
+        synth.write_model(g + ".partial", pre)
+        os.replace(g + ".partial", g)
+    return g
+
+
+def _dadizen_models(size: str, cache: str) -> Dict[str, str]:
+    """Two equal layers of one mixer kind each: windowed attention (window = the size's chunk),
+    latent attention (kv latent 4 head widths, rotated part half a head width, query latent 12 head
+    widths: the proportions of the published latent-attention models), retention (half the heads
+    at twice the value width, so the projections keep the attention layers' parameter count)."""
+    from ..models import synth
+    s = SIZES[size]
+    out = {}
+    for kind in ("attention", "latent_attention", "retention"):
+        p = os.path.join(cache, f"dadizen-{size}-{kind}")
+        if not os.path.exists(os.path.join(p, "model.safetensors")):
+            kw = dict(heads=s["heads"], kv_heads=s["kv"], dim=s["dim"], vdim=s["dim"])
+            if kind == "retention":
+                kw = dict(heads=s["heads"] // 2, dim=s["dim"], vdim=2 * s["dim"])
+            synth.write_dadizen(p, width=s["width"], kinds=(kind, kind), window=s["chunk"], rot_dim=s["dim"] // 2,
+                                q_rank=min(12 * s["dim"], s["width"]), kv_rank=4 * s["dim"], ff=s["ff"],
+                                side_dim=s["dim"], vocab=VOCAB, **kw)
+        out[f"dadizen-{kind}"] = p
+    out["llama-dense"] = _llama(size, cache)
+    return out
 
 
 def _models(size: str, cache: str) -> Dict[str, str]:
@@ -135,15 +173,15 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
 
 def run(design: str, sizes: List[str], cache: str, n_seq: int = 4, prompt: int = 2048, batch: int = 64,
         context: int = 1536, iters: int = 5) -> dict:
-    if design != "suganex":
-        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex)")
+    if design not in ("suganex", "dadizen"):
+        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex, dadizen)")
     os.makedirs(cache, exist_ok=True)
     res = {"design": design, "dtype": "bf16", "data": "synthetic", "layers": 2,
            "workload": {"prefill": f"{n_seq} x {prompt} tokens", "decode": f"batch {batch} at context {context}"},
            "sizes": {}}
     for size in sizes:
         t0 = time.time()
-        paths = _models(size, cache)
+        paths = _models(size, cache) if design == "suganex" else _dadizen_models(size, cache)
         row = {}
         for name, p in paths.items():
             row[name] = {k: round(v, 3 if k.endswith("ms") else 1)
