@@ -165,7 +165,7 @@ class _Layer:
 
 class DadizenModel:
     # what this family launches from ops/csrc (ops.require_kernels: a first run compiles only these)
-    kernel_sources = ("elementwise.hip", "norm_chain.hip", "rope_pages.hip", "retention.hip", "attention_mix.hip",
+    kernel_sources = ("elementwise.hip", "norm_chain.hip", "rope_pages.hip", "retention.hip", "attention_mix.hip", "attention_latent.hip",
                       "sampling.hip", "decode_loop.hip", "gemm_skinny.hip")
     stateful = True         # retention state per sequence: state slots, no prefix-cache reuse
     mixed_batches = True    # prompt portions and decode rows of different sequences in one forward
@@ -340,7 +340,7 @@ class DadizenModel:
         return ops.attn_mix(q, kv.k[run], kv.v[run], row_seq, fb.pos, fb.block_tables, m.heads, m.scale,
                             window=m.window, tiles=tiles, tile_rows=tile_rows, cu_q=cu_q, key_splits=splits)
 
-    def _latent(self, L: _Layer, m: MixSpec, xn, fb, kv, run, row_seq):
+    def _latent(self, L: _Layer, m: MixSpec, xn, fb, kv, run, row_seq, splits: int = 1):
         T, H, r, dn, dr = xn.shape[0], m.heads, m.kv_rank, m.dim, m.rot_dim
         proj = self._dense(ops.linear(xn, L.win))                     # [T, q_rank | kv_rank + dr | H]
         cq = self._rms(proj[:, :m.q_rank], L.dq_norm)
@@ -353,7 +353,7 @@ class DadizenModel:
         qf[:, :, :r] = torch.bmm(q[:, :, :dn].transpose(0, 1), L.uk).transpose(0, 1)
         qf[:, :, r:] = q[:, :, dn:]
         a = ops.attn_mix(qf.view(T, H * (r + dr)), kv.k[run], None, row_seq, fb.pos, fb.block_tables, H, m.scale,
-                         gate=proj[:, m.q_rank + r + dr:], v_width=r)
+                         gate=proj[:, m.q_rank + r + dr:], v_width=r, key_splits=splits)
         # ... and the value up-projection to the output side: sum_j p_j W_uv c_j = W_uv sum_j p_j c_j
         return torch.bmm(a.view(T, H, r).transpose(0, 1), L.uv_t).transpose(0, 1).reshape(T, H * m.vdim)
 
@@ -409,7 +409,7 @@ class DadizenModel:
             if m.kind == "attention":
                 a = self._attention(L, m, xn, fb, kv, r, row_seq, cu_q, tiles, tile_rows, splits_for(m))
             elif m.kind == "latent_attention":
-                a = self._latent(L, m, xn, fb, kv, r, row_seq)
+                a = self._latent(L, m, xn, fb, kv, r, row_seq, splits_for(m))
             else:
                 a = self._retention(L, m, xn, fb, kv, r, cu_q, fb.sslots)
             o = ops.linear(a, L.wo)

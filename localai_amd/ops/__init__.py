@@ -124,6 +124,7 @@ def lib():
             "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, I, P, P, I, P],
             "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
             "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, P],
+            "la_attn_latent": [P, P, P, P, P, I, I, I, I, I, I, F, I, P, I, P, I, P, P, P],
             "la_norm_chain": [P, I, I, P, I, LNG, I, I, F, P, P, F, P, I, I, F, P, P, P, I, P],
             "la_glu_clamp": [P, I, LNG, I, I, I, F, F, P, I, P],
             "la_side_gate": [P, I, LNG, I, I, I, P, P, I, I, P, I, P],
@@ -1860,7 +1861,9 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     tile's keys to that many workgroups and merges their partial results in a second launch: for
     batches of few rows with many keys each (decoding).
     v_cache None with v_width > 0: a key row's first v_width columns are also its value (latent
-    caches, where one stored row serves as key and value); such calls run on the row kernel."""
+    caches, where one stored row serves as key and value); in bf16 with one kv head, key width % 32
+    and value width % 16 such calls run on the latent matrix-core kernel (key_splits as above),
+    else on the row kernel."""
     T = q.shape[0]
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     if v_cache is None:
@@ -1922,6 +1925,22 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
         ldg = gate.stride(0)
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
     r0 = 0
+    if (v_cache is None and not f32 and G == 1 and ATTN_MIX_TILES and softcap == 0.0 and slopes is None and talk is None
+            and chunk == 0 and _has("la_attn_latent")):
+        # latent caches in bf16: the heads of a token are the rows of a matrix-core tile, the cached
+        # rows of a key tile staged once for Q.K^T and P.V (attention_latent.hip)
+        ns = max(1, min(int(key_splits), 64))
+        po = pml = None
+        if ns > 1:
+            po = torch.empty(T * H * ns * Dv, dtype=torch.float32, device=q.device)
+            pml = torch.empty(T * H * ns * 2, dtype=torch.float32, device=q.device)
+        rc = lib().la_attn_latent(q.data_ptr(), k_cache.data_ptr(), row_seq.data_ptr(), pos.data_ptr(),
+                                  block_tables.data_ptr(), block_tables.shape[1], T, H, Dk, Dv, BS, float(scale), int(window),
+                                  _ptr(gate), ldg, out.data_ptr(), ns, _ptr(po), _ptr(pml), _stream())
+        if rc == 0:
+            return out
+        if rc != 1:
+            _check(rc, "la_attn_latent")
     if (tiles is not None and tile_rows > 0 and not f32 and ATTN_MIX_TILES and Dk % 32 == 0 and Dv % 16 == 0
             and Dv <= 128 and H <= 32 and v_cache is not None):
         if cu_q is None or tile_rows > T or tiles.dtype != torch.int32 or not tiles.is_contiguous():

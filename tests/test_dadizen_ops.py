@@ -286,15 +286,22 @@ def test_window_edges_on_the_matrix_core_tiles(window):
 
 
 # --------------------------------------------------------------------------------------- latent attention, alone
+# (heads, dim, rot_dim, vdim, q_rank, kv_rank): small odd widths; widths the bf16 matrix-core kernel takes
+# (cached row % 32, latent % 16) with more heads than one 16-row tile and a head count that fills no tile
+LATENT_SHAPES = [(3, 6, 4, 5, 7, 12), (20, 16, 32, 8, 24, 96), (6, 32, 16, 16, 40, 48)]
+
+
 @pytest.mark.parametrize("device,dtype", MODES)
-def test_latent_attention_alone_with_a_far_key(device, dtype, tmp_path):
+@pytest.mark.parametrize("shape", LATENT_SHAPES)
+def test_latent_attention_alone_with_a_far_key(device, dtype, shape, tmp_path):
     """The model's latent mixer on its own (one-layer checkpoint, crafted mixer input): the cached row
     is the only thing kept per token, the up-projections act on queries and outputs."""
     import test_dadizen as td
     from localai_amd.models.dadizen import DadizenModel
     from localai_amd.models.hf_checkpoint import open_model
     cfg = {"vocab": 20, "width": 24, "norm": {"eps": 1e-5}, "layers": [
-        td.ff(td.latent(heads=3, dim=6, rot_dim=4, vdim=5, q_rank=7, kv_rank=12, scale=0.5), 0)]}
+        td.ff(td.latent(heads=shape[0], dim=shape[1], rot_dim=shape[2], vdim=shape[3], q_rank=shape[4], kv_rank=shape[5],
+                        scale=0.25), 0)]}
     Wb = td.make_weights(cfg, 11)
     td.write_checkpoint(str(tmp_path), cfg, Wb)
     W = {k: v.float() for k, v in Wb.items()}
@@ -315,6 +322,7 @@ def test_latent_attention_alone_with_a_far_key(device, dtype, tmp_path):
     for a, b in [(0, 2), (2, 150), (150, 153)] + [(t, t + 1) for t in range(153, n)]:
         pos = i32(np.arange(a, b), device)
         fb = ForwardBatch(tokens=pos, pos=pos, slots=i32(slots[a:b], device), decode=False, block_tables=i32([table], device))
-        o = model._latent(L, m, h[a:b].to(device=device, dtype=dtype), fb, kv, 0, i32(np.zeros(b - a), device))
+        o = model._latent(L, m, h[a:b].to(device=device, dtype=dtype), fb, kv, 0, i32(np.zeros(b - a), device),
+                          splits=3 if b - a == 1 else 1)     # single rows: keys dealt to three workgroups and merged
         got[a:b] = model._dense(ops.linear(o.contiguous(), L.wo)).float().cpu()
     assert rel(got, want) < (1e-4 if dtype == torch.float32 else 4e-2)
