@@ -130,7 +130,7 @@ def lib():
             "la_side_gate": [P, I, LNG, I, I, I, P, P, I, I, P, I, P],
             "la_rope_pages": [I, P, I, I, I, I, I, I, P, P, P, F, I, I, I, P, P, P, I, P],
             "la_latent_kv": [I, P, I, I, I, P, F, P, P, P, F, I, P, I, P],
-            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P],
+            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
             "la_img_resample_v_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P, P, P, P, P],
         }
@@ -2305,11 +2305,13 @@ def retention(src: torch.Tensor, H: int, Dk: int, Dv: int, pos: torch.Tensor, cu
     for t in (pos, cu_q, sslots):
         assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
     assert decay.dtype == torch.float32 and freqs.dtype == torch.float32
+    qk = torch.empty(T, 2 * Cq, dtype=torch.float32, device=src.device)      # rotated q | scaled rotated k
     o = torch.empty(T, Cv, dtype=torch.float32, device=src.device)
     out = torch.empty(T, Cv, dtype=src.dtype, device=src.device)
     _check(lib().la_retention(int(src.dtype == torch.float32), src.data_ptr(), T, nseq, H, Dk, Dv, pos.data_ptr(),
                               cu_q.data_ptr(), sslots.data_ptr(), state.data_ptr(), state.shape[0], decay.data_ptr(),
-                              freqs.data_ptr(), float(mag), rot, float(eps), o.data_ptr(), out.data_ptr(), _stream()),
+                              freqs.data_ptr(), float(mag), rot, float(eps), qk.data_ptr(), o.data_ptr(), out.data_ptr(),
+                              _stream()),
            "la_retention")
     return out
 

@@ -148,6 +148,24 @@ __global__ __launch_bounds__(256) void glu_clamp_kernel(RowSrc src, int F, long 
   put(out, out_f32, e, g / (1.f + expf(-slope * g)) * (u + 1.f));
 }
 
+// one bf16 matrix source, F % 8 == 0: 8 columns per thread, 16-byte loads and stores
+__global__ __launch_bounds__(256) void glu_clamp8_kernel(const bf16* __restrict__ src, int F, float limit, float slope,
+                                                         bf16* __restrict__ out) {
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= F) return;
+  const bf16x8 gv = *(const bf16x8*)(src + (long)t * 2 * F + c);
+  const bf16x8 uv = *(const bf16x8*)(src + (long)t * 2 * F + F + c);
+  bf16x8 ob;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float g = fminf((float)gv[j], limit);
+    const float u = fminf(fmaxf((float)uv[j], -limit), limit);
+    ob[j] = (bf16)(g / (1.f + __expf(-slope * g)) * (u + 1.f));
+  }
+  *(bf16x8*)(out + (long)t * F + c) = ob;
+}
+
 LA_DEV float gelu_tanh_f(float x) { return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x))); }
 
 __global__ __launch_bounds__(256) void side_gate_kernel(RowSrc src, int n, long total, const int* __restrict__ tok,
@@ -191,6 +209,11 @@ extern "C" int la_glu_clamp(const void* sp, int src_f32, long slab, int S, int T
                             void* out, int out_f32, void* stream) {
   using namespace la;
   if (T <= 0 || F <= 0 || !sp || !out) return -1;
+  if (!src_f32 && !out_f32 && (F & 7) == 0) {
+    hipLaunchKernelGGL(glu_clamp8_kernel, dim3(T, (F / 8 + 255) / 256), dim3(256), 0, (hipStream_t)stream, (const bf16*)sp, F,
+                       limit, slope, (bf16*)out);
+    return (int)hipGetLastError();
+  }
   RowSrc s{sp, src_f32, slab, S};
   const long total = (long)T * F;
   hipLaunchKernelGGL(glu_clamp_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, s, F,
