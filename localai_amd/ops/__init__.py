@@ -130,7 +130,7 @@ def lib():
             "la_side_gate": [P, I, LNG, I, I, I, P, P, I, I, P, I, P],
             "la_rope_pages": [I, P, I, I, I, I, I, I, P, P, P, F, I, I, I, P, P, P, I, P],
             "la_latent_kv": [I, P, I, I, I, P, F, P, P, P, F, I, P, I, P],
-            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P, P],
+            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P, P, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
             "la_img_resample_v_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P, P, P, P, P],
         }
@@ -2255,6 +2255,9 @@ def latent_kv(src: torch.Tensor, rank: int, norm_w: torch.Tensor, eps: float, po
                               int(interleaved), k_cache.data_ptr(), k_cache.shape[2], _stream()), "la_latent_kv")
 
 
+RETENTION_SEG = 128   # rows per segment of a segmented scan (retention.hip RT_SEG)
+
+
 def retention_state(slots: int, H: int, Dk: int, Dv: int, device=None) -> torch.Tensor:
     """State pool of ops.retention: fp32 [slots, H, Dv, Dk], every head's Dk x Dv state stored
     value-column major (a column's Dk entries contiguous: the kernel's threads own columns)."""
@@ -2308,10 +2311,13 @@ def retention(src: torch.Tensor, H: int, Dk: int, Dv: int, pos: torch.Tensor, cu
     qk = torch.empty(T, 2 * Cq, dtype=torch.float32, device=src.device)      # rotated q | scaled rotated k
     o = torch.empty(T, Cv, dtype=torch.float32, device=src.device)
     out = torch.empty(T, Cv, dtype=src.dtype, device=src.device)
+    # long batches scan their portions in segments of RETENTION_SEG rows: room for every segment's state
+    seg = torch.empty((T // RETENTION_SEG + nseq) * H * Dv * Dk, dtype=torch.float32, device=src.device) \
+        if T >= 8 * RETENTION_SEG else None
     _check(lib().la_retention(int(src.dtype == torch.float32), src.data_ptr(), T, nseq, H, Dk, Dv, pos.data_ptr(),
                               cu_q.data_ptr(), sslots.data_ptr(), state.data_ptr(), state.shape[0], decay.data_ptr(),
                               freqs.data_ptr(), float(mag), rot, float(eps), qk.data_ptr(), o.data_ptr(), out.data_ptr(),
-                              _stream()),
+                              _ptr(seg), _stream()),
            "la_retention")
     return out
 

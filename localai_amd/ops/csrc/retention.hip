@@ -11,9 +11,9 @@
 // retention_rot_kernel: rotated q and scaled rotated k of every row, once, as fp32 [T][2][H][Dk].
 // retention_scan_kernel: workgroup = (sequence portion, head, slice of value columns).  A column's
 // Dk state entries sit in the registers of P lanes (R each, rows interleaved over the lanes, so LDS
-// and state accesses of a lane group are consecutive); tokens are staged through LDS in chunks
-// (q, k, v) and scanned in order, o_t[c] reduced over the P lanes by shuffles.  P grows (narrower
-// column slices, more workgroups) until a launch has about four workgroups per compute unit: a scan
+// and state accesses of a lane group are consecutive), C columns a thread; tokens are staged through
+// LDS in chunks (q, k, v) and scanned in order, o_t[c] reduced over the P lanes by shuffles.  P grows
+// (narrower column slices, more workgroups) until a launch has about four workgroups per compute unit: a scan
 // is a chain of dependent steps, so it is the number of resident waves that hides its latencies.  A
 // decode batch is the same launch with one-token portions: it then streams each state once, which is
 // its memory bound.  retention_out_kernel: the per-head unit norm and the gate.
@@ -23,6 +23,8 @@ namespace la {
 
 constexpr int RT_NT = 256;
 constexpr int RT_TC = 16;     // tokens staged per chunk
+constexpr int RT_SEG = 128;   // rows per segment of a segmented portion
+enum { RT_WHOLE = 0, RT_LOCAL = 1, RT_FINAL = 2 };
 
 // qk[t][0][h][d] = rotated q, qk[t][1][h][d] = rotated k * kscale (fp32): a thread per (row, head, pair or plain dim)
 template <typename AT>
@@ -56,31 +58,55 @@ __global__ __launch_bounds__(256) void retention_rot_kernel(const AT* __restrict
   }
 }
 
-template <typename AT, int R>
+template <typename AT, int R, int C, bool EMIT>
 __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
     const AT* __restrict__ src, int ld, const float* __restrict__ qk, int H, int Dk, int Dv, const int* __restrict__ pos,
     const int* __restrict__ cu_q, const int* __restrict__ sslots, float* __restrict__ state,
-    const float* __restrict__ decay, float* __restrict__ o, int P) {
+    const float* __restrict__ decay, float* __restrict__ o, int P, int mode, int L, int maxseg,
+    float* __restrict__ seg_state) {
   extern __shared__ float lds[];
   const int DkP = P * R;                 // padded key width (rows beyond Dk hold zeros)
-  const int cpw = RT_NT / P;             // value columns of this workgroup
+  const int cpw = RT_NT / P * C;         // value columns of this workgroup
   float* qs = lds;                       // [TC][DkP]
   float* ks = qs + RT_TC * DkP;          // [TC][DkP]
   float* vs = ks + RT_TC * DkP;          // [TC][cpw]
-  const int seq = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * cpw;
-  const int tid = threadIdx.x, part = tid % P, cl = tid / P, c = c0 + cl;
-  const int a = cu_q[seq], b = cu_q[seq + 1];
-  if (b <= a) return;
-  const int slot = sslots[seq];
-  const float dec = decay[h];
-  float S[R];
-  float* st = (slot >= 0 && c < Dv) ? state + (((long)slot * H + h) * Dv + c) * Dk : nullptr;
-  const bool fresh = pos[a] == 0;
-#pragma unroll
-  for (int j = 0; j < R; ++j) {
-    const int r = j * P + part;
-    S[j] = (st && !fresh && r < Dk) ? st[r] : 0.f;
+  const int h = blockIdx.y, c0 = blockIdx.z * cpw;
+  const int tid = threadIdx.x, part = tid % P, cg = tid / P, cb = c0 + cg * C;   // this thread's first column
+  // mode RT_WHOLE: a workgroup scans a whole portion, slot state in and out.  Segmented portions:
+  // RT_LOCAL scans a segment of L rows from a zero state and leaves its end state in seg_state (no
+  // outputs, EMIT false); after retention_join_kernel has turned those into every segment's START
+  // state, RT_FINAL scans the segment again from it and writes the outputs.
+  int seq = blockIdx.x, a, b;
+  float* st = nullptr;                   // state of column cb: [C][Dk]
+  bool zero = true;
+  if (mode == RT_WHOLE) {
+    a = cu_q[seq];
+    b = cu_q[seq + 1];
+    if (b <= a) return;
+    const int slot = sslots[seq];
+    if (slot >= 0) st = state + (((long)slot * H + h) * Dv + cb) * Dk;
+    zero = pos[a] == 0;
+  } else {
+    seq = blockIdx.x / maxseg;
+    const int sidx = blockIdx.x - seq * maxseg;
+    a = cu_q[seq] + sidx * L;
+    const int b0 = cu_q[seq + 1];
+    if (a >= b0) return;
+    b = min(b0, a + L);
+    int seg = sidx;
+    for (int s2 = 0; s2 < seq; ++s2) seg += (cu_q[s2 + 1] - cu_q[s2] + L - 1) / L;
+    st = seg_state + (((long)seg * H + h) * Dv + cb) * Dk;
+    zero = mode == RT_LOCAL;
   }
+  const float dec = decay[h];
+  float S[C][R];
+#pragma unroll
+  for (int ci = 0; ci < C; ++ci)
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int r = j * P + part;
+      S[ci][j] = (st && !zero && r < Dk && cb + ci < Dv) ? st[(long)ci * Dk + r] : 0.f;
+    }
   const long vcol = 2L * H * Dk + (long)h * Dv;
   for (int t0 = a; t0 < b; t0 += RT_TC) {
     const int n = min(RT_TC, b - t0);
@@ -90,10 +116,10 @@ __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
       float qv = 0.f, kv = 0.f;
       if (d < Dk) {
         const float* row = qk + ((long)(t0 + tt) * 2 * H + h) * Dk + d;
-        qv = row[0];
+        if (EMIT) qv = row[0];
         kv = row[(long)H * Dk];
       }
-      qs[e] = qv;
+      if (EMIT) qs[e] = qv;
       ks[e] = kv;
     }
     for (int e = tid; e < n * cpw; e += RT_NT) {
@@ -102,26 +128,71 @@ __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
     }
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
-      const float vv = vs[tt * cpw + cl];
+      float vv[C], acc[C];
+#pragma unroll
+      for (int ci = 0; ci < C; ++ci) {
+        vv[ci] = vs[tt * cpw + cg * C + ci];
+        acc[ci] = 0.f;
+      }
       const float* kr = ks + tt * DkP + part;
       const float* qr = qs + tt * DkP + part;
-      float acc = 0.f;
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        S[j] = fmaf(dec, S[j], kr[j * P] * vv);
-        acc = fmaf(S[j], qr[j * P], acc);
-      }
-      for (int w = P >> 1; w > 0; w >>= 1) acc += __shfl_xor(acc, w, 64);
-      if (part == 0 && c < Dv) o[(long)(t0 + tt) * H * Dv + (long)h * Dv + c] = acc;
-    }
-  }
-  if (st) {
+        const float kj = kr[j * P];
+        const float qj = EMIT ? qr[j * P] : 0.f;
 #pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const int r = j * P + part;
-      if (r < Dk) st[r] = S[j];
+        for (int ci = 0; ci < C; ++ci) {
+          S[ci][j] = fmaf(dec, S[ci][j], kj * vv[ci]);
+          if (EMIT) acc[ci] = fmaf(S[ci][j], qj, acc[ci]);
+        }
+      }
+      if (EMIT) {
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) {
+          float v = acc[ci];
+          for (int w = P >> 1; w > 0; w >>= 1) v += __shfl_xor(v, w, 64);
+          if (part == 0 && cb + ci < Dv) o[(long)(t0 + tt) * H * Dv + (long)h * Dv + cb + ci] = v;
+        }
+      }
     }
   }
+  if (st && mode != RT_FINAL) {
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci)
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const int r = j * P + part;
+        if (r < Dk && cb + ci < Dv) st[(long)ci * Dk + r] = S[ci][j];
+      }
+  }
+}
+
+// Segment end states (from zero) -> segment start states, in place, and the portion's end state into
+// its slot:  S_start(0) = slot state (zero at position 0),  S_start(s + 1) = decay^len(s) S_start(s) + S_local(s).
+// A thread per state element of a (sequence, head).
+__global__ __launch_bounds__(256) void retention_join_kernel(const int* __restrict__ pos, const int* __restrict__ cu_q,
+                                                             const int* __restrict__ sslots, float* __restrict__ state,
+                                                             const float* __restrict__ decay, int H, long per_head,
+                                                             int L, float* __restrict__ seg_state) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const long e = (long)blockIdx.z * 256 + threadIdx.x;
+  if (e >= per_head) return;
+  const int a = cu_q[seq], n = cu_q[seq + 1] - a;
+  if (n <= 0) return;
+  int seg = 0;
+  for (int s2 = 0; s2 < seq; ++s2) seg += (cu_q[s2 + 1] - cu_q[s2] + L - 1) / L;
+  const int slot = sslots[seq];
+  float* st = slot >= 0 ? state + ((long)slot * H + h) * per_head + e : nullptr;
+  float S = (st && pos[a] != 0) ? *st : 0.f;
+  const float dec = decay[h], decL = powf(dec, (float)L);
+  for (int s = 0; s * L < n; ++s) {
+    const int len = min(L, n - s * L);
+    float* p = seg_state + ((long)(seg + s) * H + h) * per_head + e;
+    const float local = *p;
+    *p = S;
+    S = fmaf(len == L ? decL : powf(dec, (float)len), S, local);
+  }
+  if (st) *st = S;
 }
 
 // out[t][h][:] = o / sqrt(mean(o^2) + eps) * silu(gate): a wave per (token, head)
@@ -149,38 +220,65 @@ __global__ __launch_bounds__(256) void retention_out_kernel(const float* __restr
 template <typename AT>
 static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, int Dv, const int* pos, const int* cu_q,
                        const int* sslots, float* state, const float* decay, const float* freqs, float mag, int rot,
-                       float* qk, float* o, hipStream_t st) {
+                       float* qk, float* o, float* seg, hipStream_t st) {
   const float kscale = 1.f / sqrtf((float)Dk);
   {
     const long total = (long)T * H * (Dk - (rot >> 1));
     hipLaunchKernelGGL(retention_rot_kernel<AT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, src, ld, H, Dk, pos,
                        freqs, mag, rot, kscale, qk, total);
   }
-  // P lanes per value column (power of two), R rows per lane: P * R >= Dk with R <= 32; more lanes per
-  // column while the launch has fewer than about four workgroups per compute unit
+  // long batches of portions are cut into segments of RT_SEG rows scanned in parallel (two scans and a
+  // join instead of one chain of T dependent steps); seg: [T / RT_SEG + nseq][H][Dv][Dk] fp32
+  const bool segmented = seg != nullptr && T >= 8 * RT_SEG;
+  const int maxseg = (T + RT_SEG - 1) / RT_SEG;
+  const long chains = segmented ? (long)T / RT_SEG : nseq;
+  // P lanes per group of C value columns (power of two), R rows per lane: P * R >= Dk with R <= 32; a
+  // thread keeps C x R state entries, so a k / q value read from LDS feeds C multiply-adds (LDS
+  // bandwidth bounds the scan otherwise).  More lanes per group while the launch has fewer than about
+  // four workgroups per compute unit.
+  const int Cc = Dv >= 64 ? 4 : 1;
   int P = 8;
-  while (P < 64 && (Dk + P - 1) / P > 32) P <<= 1;
+  while (P < 64 && (Dk + P - 1) / P > (Cc == 4 ? 16 : 32)) P <<= 1;
   if ((Dk + P - 1) / P > 32) return -5;
-  while (P < 64 && (Dk + P - 1) / P > 2 && (long)nseq * H * ((Dv + RT_NT / P - 1) / (RT_NT / P)) < 1024) P <<= 1;
+  while (P < 64 && (Dk + P - 1) / P > 2 && chains * H * ((Dv + RT_NT / P * Cc - 1) / (RT_NT / P * Cc)) < 1024) P <<= 1;
   const int need = (Dk + P - 1) / P;
-  const int cpw = RT_NT / P;
-  dim3 grid(nseq, H, (Dv + cpw - 1) / cpw);
-#define LA_RT_LAUNCH(RR)                                                                                              \
+  const int cpw = RT_NT / P * Cc;
+  const int nz = (Dv + cpw - 1) / cpw;
+#define LA_RT_LAUNCH(RR, CC, EM, MODE, GX)                                                                            \
   {                                                                                                                   \
     const size_t shm = (size_t)(2 * RT_TC * P * RR + RT_TC * cpw) * sizeof(float);                                    \
     if (shm > 150 * 1024) return -6;                                                                                  \
     if (shm > 48 * 1024)                                                                                              \
-      (void)hipFuncSetAttribute((const void*)retention_scan_kernel<AT, RR>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                (int)shm);                                                                            \
-    hipLaunchKernelGGL((retention_scan_kernel<AT, RR>), grid, dim3(RT_NT), shm, st, src, ld, (const float*)qk, H, Dk, \
-                       Dv, pos, cu_q, sslots, state, decay, o, P);                                                    \
+      (void)hipFuncSetAttribute((const void*)retention_scan_kernel<AT, RR, CC, EM>,                                   \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                                \
+    hipLaunchKernelGGL((retention_scan_kernel<AT, RR, CC, EM>), dim3(GX, H, nz), dim3(RT_NT), shm, st, src, ld,       \
+                       (const float*)qk, H, Dk, Dv, pos, cu_q, sslots, state, decay, o, P, MODE, RT_SEG, maxseg, seg);  \
   }
-  if (need <= 1) LA_RT_LAUNCH(1)
-  else if (need <= 2) LA_RT_LAUNCH(2)
-  else if (need <= 4) LA_RT_LAUNCH(4)
-  else if (need <= 8) LA_RT_LAUNCH(8)
-  else if (need <= 16) LA_RT_LAUNCH(16)
-  else LA_RT_LAUNCH(32)
+#define LA_RT_R(CC, EM, MODE, GX)                                                                                     \
+  {                                                                                                                   \
+    if (need <= 1) LA_RT_LAUNCH(1, CC, EM, MODE, GX)                                                                  \
+    else if (need <= 2) LA_RT_LAUNCH(2, CC, EM, MODE, GX)                                                             \
+    else if (need <= 4) LA_RT_LAUNCH(4, CC, EM, MODE, GX)                                                             \
+    else if (need <= 8) LA_RT_LAUNCH(8, CC, EM, MODE, GX)                                                             \
+    else if (need <= 16) LA_RT_LAUNCH(16, CC, EM, MODE, GX)                                                           \
+    else LA_RT_LAUNCH(32, CC, EM, MODE, GX)                                                                           \
+  }
+#define LA_RT_SCAN(EM, MODE, GX)                                                                                      \
+  {                                                                                                                   \
+    if (Cc == 4) LA_RT_R(4, EM, MODE, GX)                                                                             \
+    else LA_RT_R(1, EM, MODE, GX)                                                                                     \
+  }
+  if (!segmented) {
+    LA_RT_SCAN(true, RT_WHOLE, nseq)
+    return (int)hipGetLastError();
+  }
+  LA_RT_SCAN(false, RT_LOCAL, nseq * maxseg)
+  const long per_head = (long)Dv * Dk;
+  hipLaunchKernelGGL(retention_join_kernel, dim3(nseq, H, (unsigned)((per_head + 255) / 256)), dim3(256), 0, st, pos, cu_q,
+                     sslots, state, decay, H, per_head, RT_SEG, seg);
+  LA_RT_SCAN(true, RT_FINAL, nseq * maxseg)
+#undef LA_RT_SCAN
+#undef LA_RT_R
 #undef LA_RT_LAUNCH
   return (int)hipGetLastError();
 }
@@ -189,7 +287,7 @@ static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, in
 
 extern "C" int la_retention(int f32, const void* src, int T, int nseq, int H, int Dk, int Dv, const void* pos,
                             const void* cu_q, const void* sslots, void* state, int nslots, const void* decay,
-                            const void* freqs, float mag, int rot, float eps, void* qk, void* o, void* out, void* stream) {
+                            const void* freqs, float mag, int rot, float eps, void* qk, void* o, void* out, void* seg, void* stream) {
   using namespace la;
   if (T <= 0 || nseq <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || (rot & 1) || rot > Dk || nslots <= 0) return -1;
   if (!src || !pos || !cu_q || !sslots || !state || !decay || !freqs || !qk || !o || !out) return -2;
@@ -200,14 +298,14 @@ extern "C" int la_retention(int f32, const void* src, int T, int nseq, int H, in
   if (f32) {
     rc = launch_scan<float>((const float*)src, ld, T, nseq, H, Dk, Dv, (const int*)pos, (const int*)cu_q,
                             (const int*)sslots, (float*)state, (const float*)decay, (const float*)freqs, mag, rot,
-                            (float*)qk, (float*)o, st);
+                            (float*)qk, (float*)o, (float*)seg, st);
     if (rc) return rc;
     hipLaunchKernelGGL(retention_out_kernel<float>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const float*)o,
                        (const float*)src, ld, gcol, H, Dv, rows, eps, (float*)out);
   } else {
     rc = launch_scan<bf16>((const bf16*)src, ld, T, nseq, H, Dk, Dv, (const int*)pos, (const int*)cu_q,
                            (const int*)sslots, (float*)state, (const float*)decay, (const float*)freqs, mag, rot,
-                           (float*)qk, (float*)o, st);
+                           (float*)qk, (float*)o, (float*)seg, st);
     if (rc) return rc;
     hipLaunchKernelGGL(retention_out_kernel<bf16>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const float*)o,
                        (const bf16*)src, ld, gcol, H, Dv, rows, eps, (bf16*)out);

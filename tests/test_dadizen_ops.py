@@ -216,6 +216,40 @@ def test_retention_portions_state_slots_and_reuse(device, dtype, H, Dk, Dv, rot)
         assert rel(got[s], want[s]) < (1e-4 if dtype == torch.float32 else 3e-2), s
 
 
+@pytest.mark.parametrize("device,dtype", MODES)
+def test_retention_long_portions_in_segments(device, dtype):
+    """A batch of more than a thousand rows (the GPU scans such portions in segments of 128 rows and
+    joins the segment states): portion lengths that are no multiple of the segment, one shorter than
+    a segment, a continuation from a live state, a slot with leftovers."""
+    g = torch.Generator().manual_seed(9)
+    H, Dk, Dv, rot = 2, 16, 24, 8
+    m = {"heads": H, "dim": Dk, "vdim": Dv, "decay": [1.0, 0.98], "rot": {"dims": rot, "base": 100.0}}
+    C = 2 * H * Dk + 2 * H * Dv
+    lens = {0: 700 + 300, 1: 450, 2: 60}
+    proj = {s: rounded(torch.randn(n, C, generator=g) * 0.5, dtype) for s, n in lens.items()}
+    proj[0][0, 2 * H * Dk:2 * H * Dk + Dv] *= 20          # head 0 (decay 1) carries token 0 to the end
+    eye = torch.eye(C).double()
+    Wi = {"q": eye[:H * Dk], "k": eye[H * Dk:2 * H * Dk], "v": eye[2 * H * Dk:2 * H * Dk + H * Dv],
+          "g": eye[2 * H * Dk + H * Dv:], "o": torch.eye(H * Dv).double()}
+    want = {s: oracle.retention(proj[s].double(), Wi, "", m, 1e-5) for s in lens}
+    f, mag = ops.rot_freqs(rot, 100.0, None, device)
+    state = torch.full((3, H, Dv, Dk), -3e3, dtype=torch.float32, device=device)
+    decay = torch.tensor(m["decay"], dtype=torch.float32, device=device)
+    got = {s: torch.zeros(n, H * Dv) for s, n in lens.items()}
+    for st in [[(0, 0, 700), (1, 0, 450), (2, 0, 60)], [(0, 700, 300)]]:      # 1210 rows, then 300 from the live state
+        rows = torch.cat([proj[s][a:a + n] for s, a, n in st]).to(device=device, dtype=dtype)
+        cu = np.concatenate([[0], np.cumsum([n for _, _, n in st])])
+        pos = np.concatenate([np.arange(a, a + n) for _, a, n in st])
+        out = ops.retention(rows, H, Dk, Dv, i32(pos, device), i32(cu, device), i32([s for s, _, _ in st], device), state,
+                            decay, f, rot, 1e-5, mag)
+        o = 0
+        for s, a, n in st:
+            got[s][a:a + n] = out[o:o + n].float().cpu()
+            o += n
+    for s in lens:
+        assert rel(got[s], want[s]) < (2e-4 if dtype == torch.float32 else 3e-2), s
+
+
 # --------------------------------------------------------------------------------------- windowed attention
 def _attn_case(device, dtype, H, G, Dk, Dv, rot, window, BS, n, towers, tiles):
     """rope_pages + attn_mix over shuffled pages, prompt portion then single rows, against the oracle;
