@@ -923,7 +923,8 @@ class LLMEngine:
                               slots=self._dev(plan["p_slots"]), decode=False, block_tables=self._dev(plan["p_bt"]),
                               cu_q=self._dev(cu), ctx_lens=self._dev(plan["p_ctx"]), logits_idx=idx(rows),
                               sslots=self._dev(plan["p_sslot"]),
-                              row_seq=self._dev(np.repeat(np.arange(n, dtype=np.int32), qlens)))
+                              row_seq=self._dev(np.repeat(np.arange(n, dtype=np.int32), qlens)),
+                              max_q=int(max(qlens)) if n else 0)
             # the leading portions on the tile kernel, the single-token rows after them on the row kernel
             fb.tiles, fb.tile_rows = self.model.prefill_tiles(qlens[:nc], self.device) if nc else (None, 0)
             if not rows:
@@ -995,6 +996,7 @@ class LLMEngine:
         if self.stateful:
             fb.sslots = self._dev(plan["p_sslot"])
             fb.row_seq = self._dev(np.repeat(np.arange(len(ids), dtype=np.int32), qlens))
+            fb.max_q = int(max(qlens)) if len(ids) else 0
         self.metrics["prompt_tokens"] += int(cu[-1])
         if not rows:
             self.model.forward(fb, self.kv)  # intermediate chunk: KV only

@@ -360,7 +360,7 @@ class DadizenModel:
     def _retention(self, L: _Layer, m: MixSpec, xn, fb, kv, run, cu_q, sslots):
         proj = self._dense(ops.linear(xn, L.win))                     # [T, q | k | v | gate]
         return ops.retention(proj, m.heads, m.dim, m.vdim, fb.pos, cu_q, sslots, kv.state[run], L.decay, L.freqs,
-                             m.rot.dims, self.hp.norm_eps, L.mag)
+                             m.rot.dims, self.hp.norm_eps, L.mag, max_rows=1 if fb.decode else fb.max_q)
 
     def forward(self, fb: ForwardBatch, kv: KVCache, attn_workspace=None, return_hidden: bool = False,
                 local_logits: bool = False, layer_out: Optional[list] = None) -> torch.Tensor:

@@ -225,6 +225,7 @@ class ForwardBatch:
     # (decode: of every row; -1 = none) and, for prompt batches, the sequence index of every row
     sslots: Optional[torch.Tensor] = None      # [nseq] i32 (decode: [B])
     row_seq: Optional[torch.Tensor] = None     # prefill: [T] i32
+    max_q: int = 0                             # prefill: rows of the longest portion (0: unknown)
 
 
 class KVCache:

@@ -130,7 +130,7 @@ def lib():
             "la_side_gate": [P, I, LNG, I, I, I, P, P, I, I, P, I, P],
             "la_rope_pages": [I, P, I, I, I, I, I, I, P, P, P, F, I, I, I, P, P, P, I, P],
             "la_latent_kv": [I, P, I, I, I, P, F, P, P, P, F, I, P, I, P],
-            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P, P, P],
+            "la_retention": [I, P, I, I, I, I, I, P, P, P, P, I, P, P, F, I, F, P, P, P, P, I, P],
             "la_img_resample_h": [P, I, I, P, I, P, P, I, P],
             "la_img_resample_v_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P, P, P, P, P],
         }
@@ -2266,14 +2266,16 @@ def retention_state(slots: int, H: int, Dk: int, Dv: int, device=None) -> torch.
 
 def retention(src: torch.Tensor, H: int, Dk: int, Dv: int, pos: torch.Tensor, cu_q: torch.Tensor,
               sslots: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, freqs: torch.Tensor, rot: int,
-              eps: float, mag: float = 1.0) -> torch.Tensor:
+              eps: float, mag: float = 1.0, max_rows: int = 0) -> torch.Tensor:
     """Decayed linear attention over projection rows src [T, 2 H Dk + 2 H Dv] (q | k | v | gate):
     q and k rotated on their first `rot` dims (pairs (i, i + rot / 2), angle pos * freqs[i]), k
     times Dk^-1/2; per head S <- decay_h S + k v^T, o = S^T q (no softmax, no denominator); o
     divided by its root mean square over the head (eps), times silu(gate).  Rows of a sequence
     portion are consecutive (cu_q [nseq + 1]); its state lives in state[sslots[seq]] (fp32,
     retention_state), is taken as zero when the portion starts at position 0 and advanced to the
-    portion's end.  Rotation, state, outputs and the norm are fp32.  Returns [T, H Dv] in src's dtype."""
+    portion's end.  Rotation, state, outputs and the norm are fp32.  max_rows: the longest portion
+    of the batch when the caller knows it (0: unknown, taken as T); long portions are scanned in
+    segments.  Returns [T, H Dv] in src's dtype."""
     T = src.shape[0]
     nseq = cu_q.shape[0] - 1
     Cq, Cv = H * Dk, H * Dv
@@ -2312,12 +2314,13 @@ def retention(src: torch.Tensor, H: int, Dk: int, Dv: int, pos: torch.Tensor, cu
     o = torch.empty(T, Cv, dtype=torch.float32, device=src.device)
     out = torch.empty(T, Cv, dtype=src.dtype, device=src.device)
     # long batches scan their portions in segments of RETENTION_SEG rows: room for every segment's state
+    max_rows = int(max_rows) if max_rows > 0 else T
     seg = torch.empty((T // RETENTION_SEG + nseq) * H * Dv * Dk, dtype=torch.float32, device=src.device) \
-        if T >= 8 * RETENTION_SEG else None
+        if (T >= 8 * RETENTION_SEG and max_rows >= 4 * RETENTION_SEG) else None
     _check(lib().la_retention(int(src.dtype == torch.float32), src.data_ptr(), T, nseq, H, Dk, Dv, pos.data_ptr(),
                               cu_q.data_ptr(), sslots.data_ptr(), state.data_ptr(), state.shape[0], decay.data_ptr(),
                               freqs.data_ptr(), float(mag), rot, float(eps), qk.data_ptr(), o.data_ptr(), out.data_ptr(),
-                              _ptr(seg), _stream()),
+                              _ptr(seg), max_rows, _stream()),
            "la_retention")
     return out
 

@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void retention_out_kernel(const float* __restr
 template <typename AT>
 static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, int Dv, const int* pos, const int* cu_q,
                        const int* sslots, float* state, const float* decay, const float* freqs, float mag, int rot,
-                       float* qk, float* o, float* seg, hipStream_t st) {
+                       float* qk, float* o, float* seg, int max_rows, hipStream_t st) {
   const float kscale = 1.f / sqrtf((float)Dk);
   {
     const long total = (long)T * H * (Dk - (rot >> 1));
@@ -229,8 +229,9 @@ static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, in
   }
   // long batches of portions are cut into segments of RT_SEG rows scanned in parallel (two scans and a
   // join instead of one chain of T dependent steps); seg: [T / RT_SEG + nseq][H][Dv][Dk] fp32
-  const bool segmented = seg != nullptr && T >= 8 * RT_SEG;
-  const int maxseg = (T + RT_SEG - 1) / RT_SEG;
+  // (max_rows: the longest portion of the batch, known to the host; the grid holds that many segments a sequence)
+  const bool segmented = seg != nullptr && T >= 8 * RT_SEG && max_rows >= 4 * RT_SEG;
+  const int maxseg = (max_rows + RT_SEG - 1) / RT_SEG;
   const long chains = segmented ? (long)T / RT_SEG : nseq;
   // P lanes per group of C value columns (power of two), R rows per lane: P * R >= Dk with R <= 32; a
   // thread keeps C x R state entries, so a k / q value read from LDS feeds C multiply-adds (LDS
@@ -287,7 +288,7 @@ static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, in
 
 extern "C" int la_retention(int f32, const void* src, int T, int nseq, int H, int Dk, int Dv, const void* pos,
                             const void* cu_q, const void* sslots, void* state, int nslots, const void* decay,
-                            const void* freqs, float mag, int rot, float eps, void* qk, void* o, void* out, void* seg, void* stream) {
+                            const void* freqs, float mag, int rot, float eps, void* qk, void* o, void* out, void* seg, int max_rows, void* stream) {
   using namespace la;
   if (T <= 0 || nseq <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || (rot & 1) || rot > Dk || nslots <= 0) return -1;
   if (!src || !pos || !cu_q || !sslots || !state || !decay || !freqs || !qk || !o || !out) return -2;
@@ -298,14 +299,14 @@ extern "C" int la_retention(int f32, const void* src, int T, int nseq, int H, in
   if (f32) {
     rc = launch_scan<float>((const float*)src, ld, T, nseq, H, Dk, Dv, (const int*)pos, (const int*)cu_q,
                             (const int*)sslots, (float*)state, (const float*)decay, (const float*)freqs, mag, rot,
-                            (float*)qk, (float*)o, (float*)seg, st);
+                            (float*)qk, (float*)o, (float*)seg, max_rows > 0 ? max_rows : T, st);
     if (rc) return rc;
     hipLaunchKernelGGL(retention_out_kernel<float>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const float*)o,
                        (const float*)src, ld, gcol, H, Dv, rows, eps, (float*)out);
   } else {
     rc = launch_scan<bf16>((const bf16*)src, ld, T, nseq, H, Dk, Dv, (const int*)pos, (const int*)cu_q,
                            (const int*)sslots, (float*)state, (const float*)decay, (const float*)freqs, mag, rot,
-                           (float*)qk, (float*)o, (float*)seg, st);
+                           (float*)qk, (float*)o, (float*)seg, max_rows > 0 ? max_rows : T, st);
     if (rc) return rc;
     hipLaunchKernelGGL(retention_out_kernel<bf16>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const float*)o,
                        (const bf16*)src, ld, gcol, H, Dv, rows, eps, (bf16*)out);

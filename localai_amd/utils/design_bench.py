@@ -146,6 +146,7 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
         if not dm:
             fb.sslots = eng._dev(plan["p_sslot"])
             fb.row_seq = eng._dev(np.repeat(np.arange(k, dtype=np.int32), q))
+            fb.max_q = int(max(q))
         return fb
 
     out = {}
