@@ -1862,7 +1862,7 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     batches of few rows with many keys each (decoding).
     v_cache None with v_width > 0: a key row's first v_width columns are also its value (latent
     caches, where one stored row serves as key and value); in bf16 with one kv head, key width % 32
-    and value width % 16 such calls run on the latent matrix-core kernel (key_splits as above),
+    and value width % 32 such calls run on the latent matrix-core kernel (key_splits as above),
     else on the row kernel."""
     T = q.shape[0]
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]

@@ -4,13 +4,15 @@
 // a key tile is shared by all of them:
 //
 //   workgroup = (query token, block of 16 heads[, key split]), 4 waves, per tile of 32 keys:
-//     1. the 32 cached rows -> LDS (16-byte loads through the block table), once for QK^T and PV
+//     1. the 32 cached rows -> LDS (16-byte loads through the block table, issued a tile ahead into
+//        registers), once for QK^T and PV
 //     2. S = Q K^T: MFMA 16x16x32 bf16, wave (kb, kh) = keys 16 kb.., half kh of the key width; Q
 //        fragments stay in registers over the key loop; partial sums of the two halves -> LDS
 //     3. online softmax in fp32: 16 lanes a row, two keys a lane; probabilities -> LDS as bf16 in
 //        A-operand layout, the rescale factor of the tile per row
-//     4. O += P V: wave w owns the value column blocks w, w + 4, ...; B fragments (8 keys of one
-//        column per lane) are gathered from the row-major LDS tile, which saves a transposed copy
+//     4. O += P V: wave w owns the groups of 32 value columns w, w + 4, ...; B fragments (8 keys of
+//        one column per lane) are gathered from the row-major LDS tile, which saves a transposed copy
+//        -- as dwords, two columns at once, the even and the odd columns of a group as two MFMAs
 //   epilogue: 1 / l, sigmoid head gate; with key splits the unnormalised (m, l, o) per split, merged
 //   by latent_merge_kernel.
 //
@@ -23,6 +25,7 @@ namespace la {
 constexpr int AL_KT = 32;        // keys per tile
 constexpr int AL_QF = 10;        // Q fragments a wave keeps: half of Dk / 32 <= 10  (Dk <= 640)
 constexpr int AL_NB = 8;         // value column blocks a wave owns: Dv / 16 / 4 <= 8  (Dv <= 512)
+constexpr int AL_PRE = (AL_KT * (64 * AL_QF / 8) + 255) / 256;   // 16-byte chunks of a key tile per thread
 constexpr int AL_SS = AL_KT + 1; // fp32 score row stride
 constexpr int AL_PS = AL_KT + 8; // bf16 probability row stride (16-byte aligned rows)
 
@@ -61,22 +64,46 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(
   f32x4 o[AL_NB];
 #pragma unroll
   for (int b = 0; b < AL_NB; ++b) o[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int NBT = Dv >> 4;                     // value column blocks in all
+  const int NGT = Dv >> 5;                     // groups of 32 value columns in all
   // softmax bookkeeping: thread (row srow, lanes 16) keeps the row's running max / sum in registers
   const int srow = tid >> 4, sc = tid & 15;
   float mrun = -INFINITY, lrun = 0.f;
   const int lo = window > 0 ? max(0, i - window + 1) : 0;
   const int cpr = Dk >> 3;                     // 16-byte chunks per cached row
-  for (int j0 = (lo / AL_KT + split) * AL_KT; j0 <= i; j0 += AL_KT * nsplit) {
-    __syncthreads();                           // the previous tile's PV has read ks / pb / alpha
-    // ---- 1: key tile -> LDS (rows past the query's position are zero)
-    for (int c = tid; c < AL_KT * cpr; c += 256) {
-      const int kk = c / cpr, part = c - kk * cpr;
-      const int j = j0 + kk;
+  // a tile's cached rows travel global -> registers -> LDS; the loads of the NEXT tile are issued
+  // before this tile's arithmetic, so their latency hides behind it (rows past the query are zero)
+  bf16x8 pre[AL_PRE];
+  int pkk[AL_PRE];                             // chunk u of this thread: tile row, or -1
+#pragma unroll
+  for (int u = 0; u < AL_PRE; ++u) {
+    const int c = tid + 256 * u;
+    pkk[u] = c < AL_KT * cpr ? c / cpr : -1;
+  }
+  const int bs_shift = (BS & (BS - 1)) == 0 ? __builtin_ctz(BS) : -1;
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int u = 0; u < AL_PRE; ++u) {
       bf16x8 v = {};
-      if (j <= i) v = *(const bf16x8*)(kc + ((long)tab[j / BS] * BS + j % BS) * Dk + 8 * part);
-      *(bf16x8*)(ks + kk * KS + 8 * part) = v;
+      const int kk = pkk[u], j = j0 + kk;
+      if (kk >= 0 && j <= i) {
+        const int blk = bs_shift >= 0 ? j >> bs_shift : j / BS;
+        const long slot = (long)tab[blk] * BS + (j - blk * BS);
+        v = *(const bf16x8*)(kc + slot * Dk + 8 * (tid + 256 * u - kk * cpr));
+      }
+      pre[u] = v;
     }
+  };
+  const int jfirst = (lo / AL_KT + split) * AL_KT;
+  if (jfirst <= i) fetch(jfirst);
+  for (int j0 = jfirst; j0 <= i; j0 += AL_KT * nsplit) {
+    __syncthreads();                           // the previous tile's PV has read ks / pb / alpha
+    // ---- 1: key tile -> LDS
+#pragma unroll
+    for (int u = 0; u < AL_PRE; ++u) {
+      const int kk = pkk[u];
+      if (kk >= 0) *(bf16x8*)(ks + kk * KS + 8 * (tid + 256 * u - kk * cpr)) = pre[u];
+    }
+    if (j0 + AL_KT * nsplit <= i) fetch(j0 + AL_KT * nsplit);
     __syncthreads();
     // ---- 2: partial scores of this wave's 16 keys over its half of the key width
     {
@@ -121,17 +148,27 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(
       float al[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) al[e] = alpha[4 * fq + e];
+      // value columns in groups of 32: group m = wave + 4 bp.  A lane gathers DWORDS -- columns 32 m +
+      // 2 fr and + 1 of its 8 keys -- whose low halves are the B fragment of accumulator 2 bp (the even
+      // columns of the group) and whose high halves that of 2 bp + 1 (the odd ones): half the gathers
 #pragma unroll
-      for (int b = 0; b < AL_NB; ++b) {
-        const int nb = wave + 4 * b;
-        if (nb < NBT) {
-          const bf16* vp = ks + (8 * fq) * KS + 16 * nb + fr;
-          bf16x8 vb;
+      for (int bp = 0; bp < AL_NB / 2; ++bp) {
+        const int m = wave + 4 * bp;
+        if (m < NGT) {
+          const uint32_t* vp = (const uint32_t*)(ks + (8 * fq) * KS + 32 * m) + fr;
+          uint32_t d[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) vb[e] = vp[e * KS];
+          for (int e = 0; e < 8; ++e) d[e] = vp[e * (KS >> 1)];
+          u32x4 ev, od;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o[b][e] *= al[e];
-          o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[b], 0, 0, 0);
+          for (int k = 0; k < 4; ++k) {
+            ev[k] = (d[2 * k] & 0xffffu) | (d[2 * k + 1] << 16);
+            od[k] = (d[2 * k] >> 16) | (d[2 * k + 1] & 0xffff0000u);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { o[2 * bp][e] *= al[e]; o[2 * bp + 1][e] *= al[e]; }
+          o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(bf16x8, ev), o[2 * bp], 0, 0, 0);
+          o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(bf16x8, od), o[2 * bp + 1], 0, 0, 0);
         }
       }
     }
@@ -148,9 +185,9 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(
       const long base = ((long)r * H + h) * nsplit + split;
       if (fr == 0 && wave == 0) { part_ml[2 * base] = mfin[hr]; part_ml[2 * base + 1] = lfin[hr]; }
 #pragma unroll
-      for (int b = 0; b < AL_NB; ++b) {
-        const int nb = wave + 4 * b;
-        if (nb < NBT) part_o[base * Dv + 16 * nb + fr] = o[b][e];
+      for (int bp = 0; bp < AL_NB / 2; ++bp) {
+        const int m = wave + 4 * bp;
+        if (m < NGT) *(float2*)(part_o + base * Dv + 32 * m + 2 * fr) = make_float2(o[2 * bp][e], o[2 * bp + 1][e]);
       }
       continue;
     }
@@ -158,9 +195,13 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(
     float f = l > 0.f ? 1.f / l : 0.f;
     if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)r * ldg + h]));
 #pragma unroll
-    for (int b = 0; b < AL_NB; ++b) {
-      const int nb = wave + 4 * b;
-      if (nb < NBT) out[((long)r * H + h) * Dv + 16 * nb + fr] = (bf16)(o[b][e] * f);
+    for (int bp = 0; bp < AL_NB / 2; ++bp) {
+      const int m = wave + 4 * bp;
+      if (m < NGT) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const bf16x2 pair = {(bf16)(o[2 * bp][e] * f), (bf16)(o[2 * bp + 1][e] * f)};
+        *(bf16x2*)(out + ((long)r * H + h) * Dv + 32 * m + 2 * fr) = pair;
+      }
     }
   }
 }
@@ -198,7 +239,7 @@ extern "C" int la_attn_latent(const void* q, const void* kc, const void* row_seq
                               void* out, int nsplit, void* part_o, void* part_ml, void* stream) {
   using namespace la;
   if (T <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || Dv > Dk || BS <= 0 || !q || !kc || !row_seq || !pos || !bt || !out) return -1;
-  if ((Dk & 31) || (Dv & 15) || Dk > 64 * AL_QF || Dv > 64 * AL_NB) return 1;
+  if ((Dk & 31) || (Dv & 31) || Dk > 64 * AL_QF || Dv > 64 * AL_NB) return 1;
   if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -2;
   const size_t shm = sizeof(float) * (2 * 16 * AL_SS + 48) + sizeof(bf16) * (16 * AL_PS + (size_t)AL_KT * (Dk + 8));
   if (shm > 64 * 1024) return 1;

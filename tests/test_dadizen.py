@@ -74,12 +74,13 @@ CONFIGS = {
         ff(attn(heads=2, kv=2, dim=6, vdim=6, window=7, dims=6), 20), ff(reten(heads=2, dim=4, vdim=4, dims=4), 20),
         ff(latent(heads=2, dim=4, rot_dim=4, vdim=4, q_rank=6, kv_rank=6), 20)]},
     # widths the GPU's specialised paths take: key width % 32 and value width % 16 (matrix-core
-    # attention tiles), GEMM depths % 256 (skinny GEMMs), retention rows over several registers a lane
+    # attention tiles, latent rows and cached rows % 32), GEMM depths % 256 (skinny GEMMs), retention rows over
+    # several registers a lane
     "wide": {"vocab": 97, "width": 256, "norm": {"eps": 1e-6}, "token_side": {"dim": 16}, "logit_softcap": 25.0,
              "loop": {"start": 1, "stop": 4, "times": 2}, "layers": [
                  ff(attn(heads=4, kv=2, dim=64, vdim=32, window=40, dims=32, scale=0.125), 512),
                  ff(reten(heads=2, dim=128, vdim=64, decay=(0.97, 0.995), dims=64), 0),
-                 ff(latent(heads=4, dim=32, rot_dim=16, vdim=32, q_rank=64, kv_rank=48, scale=0.14), 256),
+                 ff(latent(heads=4, dim=32, rot_dim=32, vdim=32, q_rank=48, kv_rank=64, scale=0.125), 256),
                  ff(attn(heads=8, kv=2, dim=32, vdim=16, window=24, dims=32, scale=0.18), 256)]},
 }
 

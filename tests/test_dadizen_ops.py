@@ -321,8 +321,8 @@ def test_window_edges_on_the_matrix_core_tiles(window):
 
 # --------------------------------------------------------------------------------------- latent attention, alone
 # (heads, dim, rot_dim, vdim, q_rank, kv_rank): small odd widths; widths the bf16 matrix-core kernel takes
-# (cached row % 32, latent % 16) with more heads than one 16-row tile and a head count that fills no tile
-LATENT_SHAPES = [(3, 6, 4, 5, 7, 12), (20, 16, 32, 8, 24, 96), (6, 32, 16, 16, 40, 48)]
+# (cached row % 32, latent % 32) with more heads than one 16-row tile and a head count that fills no tile
+LATENT_SHAPES = [(3, 6, 4, 5, 7, 12), (20, 16, 32, 8, 24, 96), (6, 32, 32, 16, 40, 64)]
 
 
 @pytest.mark.parametrize("device,dtype", MODES)
