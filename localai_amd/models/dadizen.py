@@ -42,7 +42,7 @@ from .decoder import ForwardBatch, KVCache, TPInfo
 
 # decode rows of softmax attention through the matrix-core tile kernel where the shape allows
 DECODE_TILES = os.environ.get("LOCALAI_AMD_DADIZEN_DECODE_TILES", "1") == "1"
-DECODE_WGS = int(os.environ.get("LOCALAI_AMD_DADIZEN_DECODE_WGS", "512"))
+DECODE_WGS = int(os.environ.get("LOCALAI_AMD_DADIZEN_DECODE_WGS", "1024"))
 
 
 @dataclass
@@ -165,8 +165,8 @@ class _Layer:
 
 class DadizenModel:
     # what this family launches from ops/csrc (ops.require_kernels: a first run compiles only these)
-    kernel_sources = ("elementwise.hip", "norm_chain.hip", "rope_pages.hip", "retention.hip", "attention_mix.hip", "attention_latent.hip",
-                      "sampling.hip", "decode_loop.hip", "gemm_skinny.hip")
+    kernel_sources = ("elementwise.hip", "norm_chain.hip", "rope_pages.hip", "retention.hip", "attention_mix.hip",
+                      "attention.hip", "attention_latent.hip", "sampling.hip", "decode_loop.hip", "gemm_skinny.hip")
     stateful = True         # retention state per sequence: state slots, no prefix-cache reuse
     mixed_batches = True    # prompt portions and decode rows of different sequences in one forward
 
@@ -298,7 +298,14 @@ class DadizenModel:
         return KVCache.layered(self._run_specs(), num_blocks, block_size, self.device, self.dtype, state_slots)
 
     def decode_workspace(self, Bp: int, ctx: int, block_size: int):
-        return None
+        """Split-KV buffers of the decode attention kernel per (heads, kv heads, width) of the layers it serves."""
+        out = {}
+        for m in self.hp.mixers:
+            if m.kind == "attention" and self._decode_kernel_ok(m, block_size):
+                key = (m.heads, m.kv_heads, m.dim)
+                if key not in out:
+                    out[key] = ops.decode_workspace(Bp, m.heads, m.kv_heads, m.dim, ctx, self.device, block_size)
+        return out or None
 
     def prefill_tiles(self, q_lens, device):
         """(16-row work tiles of the leading prompt portions for ops.attn_mix, rows they cover)."""
@@ -333,10 +340,21 @@ class DadizenModel:
         return ops.norm_chain(y, x.contiguous(), post=("rms", w, self.hp.norm_eps), pre=("cast",), replace=True,
                               out_dtype=self.dtype)
 
-    def _attention(self, L: _Layer, m: MixSpec, xn, fb, kv, run, row_seq, cu_q, tiles, tile_rows, splits):
+    def _decode_kernel_ok(self, m: MixSpec, block_size: int) -> bool:
+        """Decode batches of this layer on the framework's split-KV decode attention kernel (the llama
+        families'): bf16, equal key and value widths it is instantiated for; it takes the window."""
+        return (not self.f32 and self.device.type == "cuda" and m.dim == m.vdim and m.dim in (64, 80, 96, 128, 192, 256)
+                and m.heads // m.kv_heads <= 16 and block_size % 16 == 0 and (128 % block_size == 0 or block_size % 128 == 0)
+                and ops._has("la_attn_decode"))
+
+    def _attention(self, L: _Layer, m: MixSpec, xn, fb, kv, run, row_seq, cu_q, tiles, tile_rows, splits, ws=None):
         proj = self._dense(ops.linear(xn, L.win))
         q = ops.rope_pages(proj, m.heads, m.dim, m.kv_heads, m.dim, m.vdim, fb.pos, fb.slots, L.freqs, L.mag,
                            m.rot.dims, 0, True, kv.k[run], kv.v[run])
+        if fb.decode and fb.seq_lens is not None and self._decode_kernel_ok(m, kv.block_size):
+            T = q.shape[0]
+            return ops.attn_decode(q.view(T, m.heads, m.dim), kv.k[run], kv.v[run], fb.block_tables, fb.seq_lens, m.scale,
+                                   fb.max_len, workspace=ws, window=m.window).view(T, m.heads * m.vdim)
         return ops.attn_mix(q, kv.k[run], kv.v[run], row_seq, fb.pos, fb.block_tables, m.heads, m.scale,
                             window=m.window, tiles=tiles, tile_rows=tile_rows, cu_q=cu_q, key_splits=splits)
 
@@ -407,7 +425,8 @@ class DadizenModel:
                 y = ops.linear(torch.cat([xn, x0], 1), self.loop_in)
                 xn = nc(y, None, L.norm1, add_vec=self.loop_step[t], replace=True)
             if m.kind == "attention":
-                a = self._attention(L, m, xn, fb, kv, r, row_seq, cu_q, tiles, tile_rows, splits_for(m))
+                ws = attn_workspace.get((m.heads, m.kv_heads, m.dim)) if isinstance(attn_workspace, dict) else None
+                a = self._attention(L, m, xn, fb, kv, r, row_seq, cu_q, tiles, tile_rows, splits_for(m), ws)
             elif m.kind == "latent_attention":
                 a = self._latent(L, m, xn, fb, kv, r, row_seq, splits_for(m))
             else:

@@ -81,7 +81,7 @@ CONFIGS = {
                  ff(attn(heads=4, kv=2, dim=64, vdim=32, window=40, dims=32, scale=0.125), 512),
                  ff(reten(heads=2, dim=128, vdim=64, decay=(0.97, 0.995), dims=64), 0),
                  ff(latent(heads=4, dim=32, rot_dim=32, vdim=32, q_rank=48, kv_rank=64, scale=0.125), 256),
-                 ff(attn(heads=8, kv=2, dim=32, vdim=16, window=24, dims=32, scale=0.18), 256)]},
+                 ff(attn(heads=8, kv=2, dim=64, vdim=64, window=24, dims=32, scale=0.125), 256)]},   # decode rows: split-KV kernel
 }
 
 
