@@ -73,6 +73,12 @@ CONFIGS = {
     "plain": {"vocab": 40, "width": 24, "norm": {"eps": 1e-5}, "layers": [
         ff(attn(heads=2, kv=2, dim=6, vdim=6, window=7, dims=6), 20), ff(reten(heads=2, dim=4, vdim=4, dims=4), 20),
         ff(latent(heads=2, dim=4, rot_dim=4, vdim=4, q_rank=6, kv_rank=6), 20)]},
+    # sizes no vector load likes (width % 8 != 0, ff % 4 != 0, odd side width and ranks), three heads, a loop of one layer
+    "odd": {"vocab": 51, "width": 36, "norm": {"eps": 1e-6}, "token_side": {"dim": 5}, "logit_softcap": 12.0,
+            "loop": {"start": 2, "stop": 3, "times": 2}, "layers": [
+                ff(attn(heads=3, kv=1, dim=10, vdim=7, window=9, dims=6, scale=0.3), 30),
+                ff(reten(heads=3, dim=10, vdim=7, decay=(0.9, 0.95, 0.99), dims=10), 0),
+                ff(latent(heads=3, dim=5, rot_dim=6, vdim=7, q_rank=9, kv_rank=11), 26, 2.0)]},
     # widths the GPU's specialised paths take: key width % 32 and value width % 16 (matrix-core
     # attention tiles, latent rows and cached rows % 32), GEMM depths % 256 (skinny GEMMs), retention rows over
     # several registers a lane
@@ -212,7 +218,7 @@ def fwd(cfg, W, toks, layers_out=None):
 
 # --------------------------------------------------------------------------------------- whole prompts
 @pytest.mark.parametrize("device,dtype", MODES)
-@pytest.mark.parametrize("name", ["small", "varied", "tail", "plain", "wide"])
+@pytest.mark.parametrize("name", ["small", "varied", "tail", "plain", "odd", "wide"])
 def test_whole_prompt_matches_oracle(ckpt, name, device, dtype):
     path, cfg, W = ckpt(name)
     toks = rand_tokens(cfg, 70, 1)            # several windows of most layers, pages of 16
@@ -249,7 +255,7 @@ def test_residual_stream_after_every_layer_run(ckpt, name, device):
 
 # --------------------------------------------------------------------------------------- portions, decoding
 @pytest.mark.parametrize("device,dtype", MODES)
-@pytest.mark.parametrize("name", ["varied", "tail", "wide"])
+@pytest.mark.parametrize("name", ["varied", "tail", "odd", "wide"])
 def test_portions_and_token_by_token_decoding(ckpt, name, device, dtype):
     path, cfg, W = ckpt(name)
     toks = rand_tokens(cfg, 90, 3)
