@@ -210,23 +210,29 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(
 __global__ __launch_bounds__(128) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                            int nsplit, int H, int Dv, const bf16* __restrict__ gate, int ldg,
                                                            bf16* __restrict__ out) {
-  const int row = blockIdx.x, h = blockIdx.y;
+  __shared__ float ws[64];               // weight of every split, e^(m_s - M) / L (times the gate): nsplit <= 64
+  __shared__ float red[2];
+  const int row = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const long base = ((long)row * H + h) * nsplit;
-  float M = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
-  float L = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float m = part_ml[2 * (base + s)];
-    if (m != -INFINITY) L = fmaf(part_ml[2 * (base + s) + 1], __expf(m - M), L);
-  }
-  float f = L > 0.f ? 1.f / L : 0.f;
-  if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)row * ldg + h]));
-  for (int d = threadIdx.x; d < Dv; d += 128) {
-    float acc = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float m = part_ml[2 * (base + s)];
-      if (m != -INFINITY) acc = fmaf(part_o[(base + s) * Dv + d], __expf(m - M), acc);
+  float m = -INFINITY, l = 0.f;
+  if (tid < nsplit) { m = part_ml[2 * (base + tid)]; l = part_ml[2 * (base + tid) + 1]; }
+  // the first wave holds every split (nsplit <= 64): its maximum and weighted sum by wave reductions
+  if (tid < 64) {
+    const float M = wave_max(m);
+    const float w = m == -INFINITY ? 0.f : __expf(m - M);
+    const float L = wave_sum(l * w);
+    ws[tid] = w;
+    if (tid == 0) {
+      float f = L > 0.f ? 1.f / L : 0.f;
+      if (gate) f *= 1.f / (1.f + __expf(-(float)gate[(long)row * ldg + h]));
+      red[0] = f;
     }
+  }
+  __syncthreads();
+  const float f = red[0];
+  for (int d = tid; d < Dv; d += 128) {
+    float acc = 0.f;
+    for (int s = 0; s < nsplit; ++s) acc = fmaf(part_o[(base + s) * Dv + d], ws[s], acc);
     out[((long)row * H + h) * Dv + d] = (bf16)(acc * f);
   }
 }
